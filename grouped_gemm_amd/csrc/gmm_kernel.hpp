@@ -1,0 +1,561 @@
+// Grouped GEMM for gfx950 (MI355X): one persistent launch, scheduler on the device.
+//
+// Replaces the reference's CUTLASS grouped kernel and its argument builders
+// (csrc/grouped_gemm.cu:38-81, 230-371; csrc/fill_arguments.cuh:34-131).
+//
+// Every workgroup first derives the same schedule from batch_sizes (prefix sums of
+// rows and of tiles, kept in LDS), then walks tiles t = id, id + grid, ... .  A tile is
+// BM x BN outputs of one group.  Operand tiles go from HBM straight into LDS
+// (buffer_load_dwordx4 ... lds, 16 bytes per lane), through a ring of STAGES buffers;
+// rows past a group's end are cut off by the buffer descriptor's size, so they
+// arrive as zeros and no lane ever touches memory outside its group.  Fragments are read
+// from LDS with ds_read_b128 where the depth dimension is contiguous in memory and
+// with the transposing ds_read_b64_tr_b16 where it is not, feed
+// v_mfma_f32_32x32x16_bf16 with fp32 accumulators, and leave as bf16 through
+// buffer stores that the descriptor clips at the group's last row.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+namespace gg {
+
+constexpr int kMaxGroups = 512;
+constexpr int kSchedCols = 12;
+
+enum : int { kNN = 0, kNT = 1, kTN = 2 };
+
+using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
+using bf16x4 = __attribute__((ext_vector_type(4))) __bf16;
+using f32x16 = __attribute__((ext_vector_type(16))) float;
+using f32x4 = __attribute__((ext_vector_type(4))) float;
+using u32x2 = __attribute__((ext_vector_type(2))) uint32_t;
+
+#define GG_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+struct GmmParams {
+  const char* a;
+  const char* b;
+  char* c;
+  const int64_t* sizes_dev;  // device-resident batch_sizes, or nullptr
+  int64_t* sched_out;        // only read by the schedule dump kernel
+  int64_t tokens;            // rows of a
+  int32_t num_groups;
+  int32_t hidden_in;
+  int32_t hidden_out;
+  int32_t group_m;  // tile rows per band of the in-group tile order
+};
+
+// Host-resident batch_sizes travel in the kernel argument block: no copy, no staging.
+struct HostSizes {
+  int32_t v[kMaxGroups];
+};
+struct NoSizes {};
+
+// What every workgroup keeps in LDS about the groups.
+struct Sched {
+  int32_t row_start[kMaxGroups + 1];   // exclusive prefix sum of rows, clipped to tokens
+  int32_t rows[kMaxGroups];            // rows of `a` the group uses
+  int32_t tile_start[kMaxGroups + 1];  // exclusive prefix sum of tiles
+};
+
+constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor size used here
+constexpr uint32_t kRsrcFlags = 0x00020000u;   // raw buffer, 32-bit data format
+
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// Descriptor of `bytes` bytes at `base`.  Both are the same in every lane; reading them
+// through the first lane tells the compiler so and keeps the descriptor in scalar registers.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  const uint64_t ub = (uint64_t)(uint32_t)uniform((int)(uint32_t)b) |
+                      ((uint64_t)(uint32_t)uniform((int)(uint32_t)(b >> 32)) << 32);
+  return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(ub), 0,
+                                           (uint32_t)uniform((int)bytes), kRsrcFlags);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ void block_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// ---------------------------------------------------------------------- schedule
+
+template <int LAYOUT, int BM, int BN>
+__device__ __forceinline__ int tiles_of_group(int rows, int hidden_in, int hidden_out) {
+  const int tiles_n = (hidden_out + BN - 1) / BN;
+  if (LAYOUT == kTN) return ((hidden_in + BM - 1) / BM) * tiles_n;
+  return ((rows + BM - 1) / BM) * tiles_n;
+}
+
+// Run by the first wave of a workgroup.  Each lane owns up to 8 consecutive groups; one
+// wave-wide scan of int64 row counts and one of int32 tile counts.
+template <int LAYOUT, int BM, int BN, bool HOST_SIZES, typename SizesArg>
+__device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, const SizesArg& hs) {
+  const int lane = threadIdx.x;
+  if (lane >= 64) return;
+  const int E = p.num_groups;
+  const int per = (E + 63) >> 6;
+  const int e0 = lane * per;
+  int64_t sz[8];
+  int64_t sum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = e0 + i;
+    int64_t v = 0;
+    if (i < per && e < E) {
+      if constexpr (HOST_SIZES) {
+        v = hs.v[e];
+      } else {
+        v = p.sizes_dev[e];
+      }
+      v = v < 0 ? 0 : v;
+    }
+    sz[i] = v;
+    sum += v;
+  }
+  int64_t incl = sum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int64_t o = __shfl_up(incl, d);
+    if (lane >= d) incl += o;
+  }
+  int64_t run = incl - sum;
+  int rows[8];
+  int tsum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = e0 + i;
+    const int64_t start = run < p.tokens ? run : p.tokens;
+    const int64_t left = p.tokens - start;
+    const int r = (int)(sz[i] < left ? sz[i] : left);
+    rows[i] = r;
+    if (i < per && e < E) {
+      s->row_start[e] = (int)start;
+      s->rows[e] = r;
+      tsum += tiles_of_group<LAYOUT, BM, BN>(r, p.hidden_in, p.hidden_out);
+    }
+    run += sz[i];
+  }
+  int tincl = tsum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int o = __shfl_up(tincl, d);
+    if (lane >= d) tincl += o;
+  }
+  int trun = tincl - tsum;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = e0 + i;
+    if (i < per && e < E) {
+      s->tile_start[e] = trun;
+      trun += tiles_of_group<LAYOUT, BM, BN>(rows[i], p.hidden_in, p.hidden_out);
+    }
+  }
+  if (lane == 63) {
+    s->row_start[E] = (int)(run < p.tokens ? run : p.tokens);
+    s->tile_start[E] = tincl;
+  }
+}
+
+// Element offsets of a group's A, B and C blocks, the quantities of the reference's
+// problem table (csrc/fill_arguments.cuh:72-76) in int64.  The kernel addresses memory
+// through these and the schedule dump prints these.
+struct GroupGeom {
+  int64_t a_off, b_off, c_off;
+  int32_t m, n, k;
+};
+
+template <int LAYOUT>
+__device__ __forceinline__ GroupGeom group_geometry(const Sched* s, const GmmParams& p, int e) {
+  GroupGeom g;
+  // read through the first lane: everything derived from these stays in scalar registers
+  const int64_t start = uniform(s->row_start[e]);
+  const int rows = uniform(s->rows[e]);
+  const int64_t hin = p.hidden_in, hout = p.hidden_out;
+  if (LAYOUT == kTN) {
+    g.m = p.hidden_in;
+    g.n = p.hidden_out;
+    g.k = rows;
+    g.a_off = hin * start;
+    g.b_off = start * hout;
+    g.c_off = (int64_t)e * hin * hout;
+  } else {
+    g.m = rows;
+    g.n = p.hidden_out;
+    g.k = p.hidden_in;
+    g.a_off = start * hin;
+    g.b_off = (int64_t)e * hin * hout;
+    g.c_off = start * hout;
+  }
+  return g;
+}
+
+// In-group tile order: bands of `group_m` tile rows, tile rows fastest inside a band, so
+// that tiles running at the same time share A rows and B columns in L2.
+__device__ __forceinline__ void tile_coords(int u, int tiles_m, int tiles_n, int group_m,
+                                            int* tm, int* tn) {
+  const int per_band = group_m * tiles_n;
+  const int band = u / per_band;
+  const int first_m = band * group_m;
+  const int left = tiles_m - first_m;
+  const int gsz = left < group_m ? left : group_m;
+  const int r = u - band * per_band;
+  *tm = first_m + r % gsz;
+  *tn = r / gsz;
+}
+
+template <int LAYOUT, int BM, int BN, bool HOST_SIZES>
+__global__ __launch_bounds__(64) void schedule_dump_kernel(
+    GmmParams p, std::conditional_t<HOST_SIZES, HostSizes, NoSizes> hs) {
+  __shared__ Sched s;
+  build_schedule<LAYOUT, BM, BN, HOST_SIZES>(&s, p, hs);
+  __syncthreads();
+  for (int e = threadIdx.x; e < p.num_groups; e += 64) {
+    const GroupGeom g = group_geometry<LAYOUT>(&s, p, e);
+    int64_t* row = p.sched_out + (int64_t)e * kSchedCols;
+    row[0] = g.m;
+    row[1] = g.n;
+    row[2] = g.k;
+    row[3] = LAYOUT == kTN ? g.m : g.k;  // lda: column-major A has ld = rows
+    row[4] = LAYOUT == kNT ? g.k : g.n;  // ldb
+    row[5] = g.n;                        // ldc
+    row[6] = g.a_off;
+    row[7] = g.b_off;
+    row[8] = g.c_off;
+    row[9] = s.tile_start[e];
+    row[10] = s.tile_start[e + 1] - s.tile_start[e];
+    row[11] = s.rows[e];
+  }
+}
+
+// ------------------------------------------------------------ operand tile movers
+//
+// Two kinds of operand tile, by which dimension is contiguous in memory.
+//
+// DepthMajor ("KC"): R rows (M or N index) of BK depth elements, depth contiguous.  LDS
+// keeps row-major rows of BK*2 bytes; the 16-byte chunk c of row r sits at chunk slot
+// c ^ ((r / RP) % CPR), which makes 16 consecutive rows at one depth hit 64 distinct
+// banks for ds_read_b128.
+//
+// WidthMajor ("MC"): BK depth rows of W elements (M or N index contiguous).  LDS keeps
+// row-major rows of W*2 bytes; 64-byte segment s of depth row k sits at segment slot
+// s ^ g(k), g(k) = (k & 3) | ((k >> 1) & 4), so the 8 depth rows one transposing read
+// touches land in distinct bank groups.
+//
+// A lane's LDS slot is fixed by the hardware (wave base + lane * 16), so the swizzle is
+// applied by choosing which global chunk each lane fetches.
+
+template <int R, int BK, int NT>
+struct DepthMajor {
+  static constexpr int CPR = BK / 8;                                  // chunks per row
+  static constexpr int RP = (BK * 2 >= 256) ? 1 : 256 / (BK * 2);     // rows per 256 B
+  static constexpr int ROWS_PER_INSTR = NT / CPR;
+  static constexpr int NI = R * CPR / NT;                             // loads per lane per tile
+  static constexpr int BYTES = R * BK * 2;
+  static_assert(NT % CPR == 0 && (R * CPR) % NT == 0, "tile does not split over the block");
+  static_assert(ROWS_PER_INSTR % (RP * CPR) == 0, "swizzle must not depend on the load index");
+
+  const char* base;   // first row of the tile, depth 0
+  int ld;             // elements between rows ( = depth extent )
+  int rows_valid;     // rows of the tile that exist
+  int depth;          // depth extent
+  int my_chunk;       // depth chunk (of 8) this lane fetches
+  uint32_t voff0;     // byte offset of this lane's chunk for load 0
+
+  __device__ __forceinline__ void setup(const char* tile_base, int ld_, int rows_valid_, int depth_) {
+    base = tile_base;
+    ld = ld_;
+    rows_valid = rows_valid_;
+    depth = depth_;
+    const int tid = threadIdx.x;
+    const int row = tid / CPR, pos = tid % CPR;
+    my_chunk = pos ^ ((row / RP) % CPR);
+    voff0 = (uint32_t)(row * ld + my_chunk * 8) * 2u;
+  }
+
+  // Fetch depth slice [kt*BK, kt*BK+BK) into the LDS tile at `dst` (wave-uniform).
+  __device__ __forceinline__ void issue(int kt, char* dst, int wave) const {
+    const int left = uniform(depth - kt * BK);
+    const uint32_t bytes = (left > 0 && rows_valid > 0)
+                               ? (uint32_t)((rows_valid - 1) * ld + left) * 2u : 0u;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)kt * (BK * 2), bytes);
+    uint32_t v = voff0;
+    if (left < BK) v = (my_chunk * 8 < left) ? v : kOutOfRange;   // depth tail, uniform branch
+    const uint32_t step = (uint32_t)(ROWS_PER_INSTR * ld) * 2u;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, GG_LDS_PTR(dst + (i * NT + wave * 64) * 16), 16,
+                                               v, 0, 0, 0);
+      v += step;
+    }
+  }
+};
+
+template <int W, int BK, int NT>
+struct WidthMajor {
+  static constexpr int CPRW = W / 8;                  // chunks per depth row
+  static constexpr int SEGS = W * 2 / 64;             // 64-byte segments per depth row
+  static constexpr int ROWS_PER_INSTR = NT / CPRW;
+  static constexpr int NI = BK * CPRW / NT;
+  static constexpr int BYTES = W * BK * 2;
+  static constexpr int PITCH = W * 2;
+  static_assert(NT % CPRW == 0 && (BK * CPRW) % NT == 0, "tile does not split over the block");
+  static_assert(SEGS >= 4, "needs at least 128 columns");
+
+  __device__ static __forceinline__ int seg_swizzle(int krow) {
+    return (krow & 3) | (SEGS >= 8 ? ((krow >> 1) & 4) : 0);
+  }
+
+  const char* base;      // depth row 0 of the group, column 0
+  int ld;                // elements between depth rows
+  int depth;             // depth rows of the group
+  uint32_t voff[NI];     // byte offset of this lane's chunk per load (kOutOfRange past the width)
+
+  __device__ __forceinline__ void setup(const char* group_base, int ld_, int depth_, int col0,
+                                        int width) {
+    base = group_base;
+    ld = ld_;
+    depth = depth_;
+    const int tid = threadIdx.x;
+    const int krow0 = tid / CPRW, p = tid % CPRW;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int krow = krow0 + i * ROWS_PER_INSTR;
+      const int c = (((p >> 2) ^ seg_swizzle(krow)) << 2) | (p & 3);
+      const int col = col0 + c * 8;
+      voff[i] = col < width ? (uint32_t)(krow * ld + col) * 2u : kOutOfRange;
+    }
+  }
+
+  __device__ __forceinline__ void issue(int kt, char* dst, int wave) const {
+    int left = uniform(depth - kt * BK);
+    left = left < 0 ? 0 : (left > BK ? BK : left);
+    const __amdgpu_buffer_rsrc_t r =
+        make_rsrc(base + (int64_t)kt * BK * ld * 2, (uint32_t)(left * ld) * 2u);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, GG_LDS_PTR(dst + (i * NT + wave * 64) * 16), 16,
+                                               voff[i], 0, 0, 0);
+    }
+  }
+};
+
+// ---------------------------------------------------------------- fragment readers
+// A fragment is the operand of one 32x32x16 MFMA: lane l holds 8 depth values
+// 8*(l/32) .. +7 of row (or column) l % 32.
+
+template <int BK>
+struct DepthMajorFrag {
+  static constexpr int CPR = BK / 8;
+  static constexpr int RP = (BK * 2 >= 256) ? 1 : 256 / (BK * 2);
+  uint32_t off[BK / 16];   // lane offset per 16-deep step, block 0
+
+  __device__ __forceinline__ void setup(int wave_row0) {
+    const int lane = threadIdx.x & 63;
+    const int row = wave_row0 + (lane & 31);
+    const int sw = (row / RP) % CPR;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      off[ks] = (uint32_t)(row * (BK * 2) + (((ks * 2 + (lane >> 5)) ^ sw) << 4));
+    }
+  }
+  __device__ __forceinline__ bf16x8 read(const char* tile, int ks, int blk) const {
+    return *reinterpret_cast<const bf16x8*>(tile + off[ks] + blk * 32 * (BK * 2));
+  }
+};
+
+template <int W, int BK, int NBLK>
+struct WidthMajorFrag {
+  static constexpr int PITCH = W * 2;
+  static constexpr int SEGS = W * 2 / 64;
+  uint32_t off[NBLK];   // lane offset per 32-wide block, depth step 0
+
+  __device__ __forceinline__ void setup(int wave_col0) {
+    const int lane = threadIdx.x & 63;
+    const int l16 = lane & 15;
+    const int krow = 8 * (lane >> 5) + (l16 >> 2);
+    const int g = (krow & 3) | (SEGS >= 8 ? ((krow >> 1) & 4) : 0);
+#pragma unroll
+    for (int j = 0; j < NBLK; ++j) {
+      const int seg = (wave_col0 >> 5) + j;
+      off[j] = (uint32_t)(krow * PITCH + ((seg ^ g) << 6) + 32 * ((lane >> 4) & 1) + 8 * (l16 & 3));
+    }
+  }
+  __device__ __forceinline__ bf16x8 read(const char* tile, int ks, int blk) const {
+    const char* p = tile + off[blk] + ks * 16 * PITCH;
+    const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (__attribute__((address_space(3))) bf16x4*)GG_LDS_PTR(p));
+    const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (__attribute__((address_space(3))) bf16x4*)GG_LDS_PTR(p + 4 * PITCH));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+};
+
+// ------------------------------------------------------------------------ kernel
+
+template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N>
+struct GmmConfig {
+  static constexpr int NT = WAVES_M * WAVES_N * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int MB = WTM / 32, NB = WTN / 32;
+  static constexpr bool A_DEPTH_MAJOR = LAYOUT != kTN;
+  static constexpr bool B_DEPTH_MAJOR = LAYOUT == kNT;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + (int)sizeof(Sched);
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
+  static_assert(BK % 16 == 0 && STAGES >= 2, "");
+};
+
+template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool HOST_SIZES>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
+    GmmParams p, std::conditional_t<HOST_SIZES, HostSizes, NoSizes> hs) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
+  using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
+  constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB;
+  using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT>, WidthMajor<BM, BK, NT>>;
+  using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT>, WidthMajor<BN, BK, NT>>;
+  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BM, BK, MB>>;
+  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BN, BK, NB>>;
+  constexpr int LOADS_PER_TILE = ALoad::NI + BLoad::NI;
+  static_assert((STAGES - 2) * LOADS_PER_TILE < 64, "too many loads in flight for vmcnt");
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  Sched* sched = reinterpret_cast<Sched*>(smem + STAGES * Cfg::STAGE_BYTES);
+  build_schedule<LAYOUT, BM, BN, HOST_SIZES>(sched, p, hs);
+  __syncthreads();
+
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  AFrag afrag;
+  BFrag bfrag;
+  afrag.setup(wm * Cfg::WTM);
+  bfrag.setup(wn * Cfg::WTN);
+
+  const int E = p.num_groups;
+  const int total_tiles = uniform(sched->tile_start[E]);
+  const int tiles_n = (p.hidden_out + BN - 1) / BN;
+  const int tiles_m_fixed = (p.hidden_in + BM - 1) / BM;   // TN only
+
+  // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
+  // tile indices so that its private L2 sees neighbouring tiles.
+  const int G = gridDim.x;
+  const int w = blockIdx.x;
+  const int vid = (G % 8 == 0) ? (w % 8) * (G / 8) + (w / 8) : w;
+
+  int e = 0;
+  for (int t = vid; t < total_tiles; t += G) {
+    while (t >= uniform(sched->tile_start[e + 1])) ++e;
+    const GroupGeom g = group_geometry<LAYOUT>(sched, p, e);
+    const int u = t - uniform(sched->tile_start[e]);
+    const int tiles_m = LAYOUT == kTN ? tiles_m_fixed : (g.m + BM - 1) / BM;
+    int tm, tn;
+    tile_coords(u, tiles_m, tiles_n, p.group_m, &tm, &tn);
+    tm = uniform(tm);
+    tn = uniform(tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int rows_valid = min(BM, g.m - m0);
+    const int depth = g.k;
+    const int nk = (depth + BK - 1) / BK;
+
+    ALoad aload;
+    BLoad bload;
+    if constexpr (Cfg::A_DEPTH_MAJOR) {
+      aload.setup(p.a + (g.a_off + (int64_t)m0 * g.k) * 2, g.k, rows_valid, depth);
+    } else {
+      aload.setup(p.a + g.a_off * 2, g.m, depth, m0, g.m);
+    }
+    if constexpr (Cfg::B_DEPTH_MAJOR) {
+      bload.setup(p.b + (g.b_off + (int64_t)n0 * g.k) * 2, g.k, min(BN, g.n - n0), depth);
+    } else {
+      bload.setup(p.b + g.b_off * 2, g.n, depth, n0, g.n);
+    }
+
+    f32x16 acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // every wave is done reading the previous tile's buffers
+    block_barrier();
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+      char* st = smem + s * Cfg::STAGE_BYTES;
+      aload.issue(s, st, wave);
+      bload.issue(s, st + Cfg::A_BYTES, wave);
+    }
+    int rd = 0, wr = STAGES - 1;
+    for (int kt = 0; kt < nk; ++kt) {
+      wait_vmcnt<(STAGES - 2) * LOADS_PER_TILE>();
+      block_barrier();
+      {
+        // slices past the depth are fetched with an empty descriptor: zeros, no traffic,
+        // and the count of loads in flight stays the same in every iteration
+        char* st = smem + wr * Cfg::STAGE_BYTES;
+        aload.issue(kt + STAGES - 1, st, wave);
+        bload.issue(kt + STAGES - 1, st + Cfg::A_BYTES, wave);
+      }
+      const char* sa = smem + rd * Cfg::STAGE_BYTES;
+      const char* sb = sa + Cfg::A_BYTES;
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ++ks) {
+        bf16x8 af[MB], bfv[NB];
+#pragma unroll
+        for (int i = 0; i < MB; ++i) af[i] = afrag.read(sa, ks, i);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) bfv[j] = bfrag.read(sb, ks, j);
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
+            // operands swapped: the result block is held transposed, so a lane owns four
+            // consecutive columns of one output row
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfv[j], af[i], acc[i][j], 0, 0, 0);
+      }
+      rd = rd + 1 == STAGES ? 0 : rd + 1;
+      wr = wr + 1 == STAGES ? 0 : wr + 1;
+    }
+    wait_vmcnt<0>();
+
+    // epilogue: lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3
+    {
+      const char* cbase = p.c + (g.c_off + (int64_t)m0 * g.n) * 2;
+      const uint32_t cbytes = rows_valid > 0 ? (uint32_t)(rows_valid * g.n) * 2u : 0u;
+      const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int row = wm * Cfg::WTM + i * 32 + (lane & 31);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int col = n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+            bf16x4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][4 * q + r];
+            const uint32_t off = col < g.n ? (uint32_t)(row * g.n + col) * 2u : kOutOfRange;
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, o), rc, off, 0, 0);
+          }
+        }
+      }
+    }
+  }
+#endif  // __HIP_DEVICE_COMPILE__
+}
+
+}  // namespace gg
