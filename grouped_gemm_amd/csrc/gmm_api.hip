@@ -148,10 +148,10 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
   int rc = check_common(batch_sizes, num_groups, tokens, hidden_in, hidden_out, trans_a, trans_b);
   if (rc != GG_OK) return rc;
   if (num_groups == 0) return GG_OK;
-  if ((tokens > 0 && (a == nullptr || (trans_a && b == nullptr))) || (!trans_a && b == nullptr) ||
-      c == nullptr)
-    if (hidden_in > 0 && hidden_out > 0) return fail(GG_EINVAL, "a, b or c is null");
-  if (hidden_out == 0 || (!trans_a && tokens == 0) || (trans_a && hidden_in == 0)) return GG_OK;
+  // nothing to write
+  if (hidden_out == 0 || (trans_a ? hidden_in == 0 : tokens == 0)) return GG_OK;
+  if (c == nullptr) return fail(GG_EINVAL, "c is null");
+  if (tokens > 0 && (a == nullptr || b == nullptr)) return fail(GG_EINVAL, "a or b is null");
   if (batch_sizes_on_device && num_groups > GG_MAX_GROUPS_PER_LAUNCH)
     return fail(GG_ELIMIT, "at most %d groups are supported when batch_sizes is on the device, got %lld",
                 GG_MAX_GROUPS_PER_LAUNCH, (long long)num_groups);

@@ -1,0 +1,138 @@
+// PyTorch-ROCm binding: module `grouped_gemm_backend`, one function
+// gmm(a, b, c, batch_sizes, trans_a, trans_b) -> None, the same entry point the
+// reference's extension exports (csrc/ops.cu:7-9, csrc/grouped_gemm.h:5-9).
+//
+// All tensor validation lives here, in the order of the reference's checks
+// (csrc/grouped_gemm.cu:470-540, :437-460, :120-124), and runs before anything touches
+// the device; the compute is one call into the C ABI of libgrouped_gemm_hip.so on
+// torch's current HIP stream.
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/extension.h>
+
+#include "../../include/grouped_gemm_hip.h"
+
+namespace grouped_gemm {
+
+namespace {
+
+// `on_device` false skips the checks that a tensor lives on the GPU, so that the shape,
+// rank and dtype rules can be exercised with CPU tensors on a machine without one.
+void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
+              const torch::Tensor& batch_sizes, bool trans_a, bool trans_b, bool on_device) {
+  // Only one of the operands may be transposed (csrc/grouped_gemm.cu:476).
+  TORCH_CHECK(!(trans_a && trans_b), "grouped_gemm: trans_a and trans_b cannot both be set");
+
+  // batch_sizes may live on the host or on the device (csrc/grouped_gemm.cu:478-486).
+  TORCH_CHECK(batch_sizes.is_cuda() || batch_sizes.is_cpu(),
+              "grouped_gemm: batch_sizes must be a CPU or GPU tensor");
+  TORCH_CHECK(batch_sizes.ndimension() == 1, "grouped_gemm: batch_sizes must be 1-d");
+  TORCH_CHECK(batch_sizes.scalar_type() == torch::kInt64, "grouped_gemm: batch_sizes must be int64");
+
+  // a: (tokens, hidden_in) bf16 on the GPU (csrc/grouped_gemm.cu:490-492).
+  if (on_device) TORCH_CHECK(a.is_cuda(), "grouped_gemm: a must be a GPU tensor");
+  TORCH_CHECK(a.ndimension() == 2, "grouped_gemm: a must be 2-d");
+  TORCH_CHECK(a.scalar_type() == torch::kBFloat16, "grouped_gemm: a must be bfloat16");
+
+  // b, c: bf16 on the GPU (csrc/grouped_gemm.cu:503-506).
+  if (on_device) {
+    TORCH_CHECK(b.is_cuda(), "grouped_gemm: b must be a GPU tensor");
+    TORCH_CHECK(c.is_cuda(), "grouped_gemm: c must be a GPU tensor");
+  }
+  TORCH_CHECK(b.scalar_type() == torch::kBFloat16, "grouped_gemm: b must be bfloat16");
+  TORCH_CHECK(c.scalar_type() == torch::kBFloat16, "grouped_gemm: c must be bfloat16");
+
+  if (trans_a) {
+    // b (tokens, hidden_out), c (num_experts, hidden_in, hidden_out)
+    // (csrc/grouped_gemm.cu:513-522).
+    TORCH_CHECK(b.ndimension() == 2, "grouped_gemm: with trans_a, b must be 2-d");
+    TORCH_CHECK(c.ndimension() == 3, "grouped_gemm: with trans_a, c must be 3-d");
+    TORCH_CHECK(b.size(0) == a.size(0), "grouped_gemm: a and b must have the same number of rows");
+    TORCH_CHECK(c.size(0) == batch_sizes.size(0), "grouped_gemm: c.size(0) must equal the number of experts");
+    TORCH_CHECK(c.size(1) == a.size(1), "grouped_gemm: c.size(1) must equal a.size(1)");
+    TORCH_CHECK(c.size(2) == b.size(1), "grouped_gemm: c.size(2) must equal b.size(1)");
+  } else {
+    // b (num_experts, hidden_in, hidden_out) or transposed, c (tokens, hidden_out)
+    // (csrc/grouped_gemm.cu:524-534).
+    TORCH_CHECK(b.ndimension() == 3, "grouped_gemm: b must be 3-d");
+    TORCH_CHECK(c.ndimension() == 2, "grouped_gemm: c must be 2-d");
+    const int64_t hidden_in = trans_b ? b.size(2) : b.size(1);
+    TORCH_CHECK(hidden_in == a.size(1), "grouped_gemm: contraction dimensions of a and b differ");
+    TORCH_CHECK(batch_sizes.size(0) == b.size(0), "grouped_gemm: need one batch size per expert");
+    // The reference leaves the shape of c unchecked here; a wrong one would make the
+    // kernel write outside c, so it is rejected.
+    const int64_t hidden_out = trans_b ? b.size(1) : b.size(2);
+    TORCH_CHECK(c.size(0) == a.size(0) && c.size(1) == hidden_out,
+                "grouped_gemm: c must have shape (tokens, hidden_out)");
+  }
+
+  // Transposition goes through the flags only (csrc/grouped_gemm.cu:538-540).
+  TORCH_CHECK(a.is_contiguous(), "grouped_gemm: a must be contiguous");
+  TORCH_CHECK(b.is_contiguous(), "grouped_gemm: b must be contiguous");
+  TORCH_CHECK(c.is_contiguous(), "grouped_gemm: c must be contiguous");
+
+  // Device-resident sizes are scheduled by one launch (csrc/grouped_gemm.cu:120-124).
+  if (batch_sizes.is_cuda()) {
+    TORCH_CHECK(batch_sizes.size(0) <= GG_MAX_GROUPS_PER_LAUNCH, "At most ", GG_MAX_GROUPS_PER_LAUNCH,
+                " experts are supported when batch_sizes is a GPU tensor, but got ",
+                batch_sizes.size(0));
+    TORCH_CHECK(batch_sizes.is_contiguous(), "grouped_gemm: batch_sizes must be contiguous");
+    if (on_device)
+      TORCH_CHECK(batch_sizes.device() == a.device(), "grouped_gemm: batch_sizes is on another GPU");
+  }
+  if (on_device) {
+    TORCH_CHECK(b.device() == a.device() && c.device() == a.device(),
+                "grouped_gemm: a, b and c must be on the same GPU");
+  }
+}
+
+}  // namespace
+
+void GroupedGemm(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes,
+                 bool trans_a, bool trans_b) {
+  Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/true);
+
+  const int64_t tokens = a.size(0);
+  const int64_t hidden_in = a.size(1);
+  const int64_t hidden_out = trans_a ? b.size(1) : (trans_b ? b.size(1) : b.size(2));
+  torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
+  const int rc = gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), sizes.data_ptr<int64_t>(),
+                             sizes.is_cuda() ? 1 : 0, sizes.size(0), tokens, hidden_in, hidden_out,
+                             trans_a ? 1 : 0, trans_b ? 1 : 0, static_cast<void*>(stream));
+  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+}
+
+// The on-device scheduler's view of the groups, as an int64 tensor
+// (num_experts, GG_SCHED_COLS) on `device`; see gg_debug_schedule.
+torch::Tensor DebugSchedule(torch::Tensor batch_sizes, int64_t tokens, int64_t hidden_in,
+                            int64_t hidden_out, bool trans_a, bool trans_b, torch::Device device) {
+  TORCH_CHECK(batch_sizes.ndimension() == 1 && batch_sizes.scalar_type() == torch::kInt64);
+  TORCH_CHECK(device.is_cuda(), "grouped_gemm: the schedule is computed on a GPU");
+  torch::Tensor sizes = batch_sizes.contiguous();
+  if (sizes.is_cuda()) TORCH_CHECK(sizes.device() == device);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(device);
+  torch::Tensor out = torch::zeros({sizes.size(0), GG_SCHED_COLS},
+                                   torch::dtype(torch::kInt64).device(device));
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index()).stream();
+  const int rc = gg_debug_schedule(sizes.data_ptr<int64_t>(), sizes.is_cuda() ? 1 : 0, sizes.size(0),
+                                   tokens, hidden_in, hidden_out, trans_a ? 1 : 0, trans_b ? 1 : 0,
+                                   out.data_ptr<int64_t>(), static_cast<void*>(stream));
+  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+  return out;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("gmm", &GroupedGemm, "Grouped GEMM.");
+  m.def("validate",
+        [](torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes, bool trans_a,
+           bool trans_b) { Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/false); },
+        "Shape, rank and dtype checks of gmm without the device checks.");
+  m.def("debug_schedule", &DebugSchedule, "Per-group table derived by the on-device scheduler.");
+  m.attr("max_groups_per_launch") = GG_MAX_GROUPS_PER_LAUNCH;
+  m.attr("sched_cols") = GG_SCHED_COLS;
+}
+
+}  // namespace grouped_gemm

@@ -1,0 +1,463 @@
+"""GPU parity tests: the HIP path against the CPU oracle.
+
+Layout of this file follows the reference's own tests (grouped_gemm/ops_test.py):
+fixed sizes, variable sizes, the zero-size expert at Mixtral shape, the zero-K known
+answer; then the five benchmark configurations, the C ABI called directly, the
+on-device schedule bit-exact against the int64 closed forms, and edge cases.
+
+Tolerance (every element): |got - want| <= 1e-2 + 1.6e-2 * |want| against the
+fp32-accumulated oracle.  Small cases use the oracle on the CPU; full-size cases run
+the oracle's per-expert loop with torch on the GPU in fp32 and add a CPU fp64 check on
+sampled rows so that no GPU library is trusted alone.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+RTOL, ATOL = 1.6e-2, 1e-2
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from grouped_gemm import ops as _ops
+    return _ops
+
+
+def _announce(*what):
+    print("[case]", *what, flush=True)
+
+
+def check(got, want, what):
+    got = got.float().cpu() if got.numel() < (1 << 24) else got.float()
+    want = want.float().to(got.device)
+    assert tuple(got.shape) == tuple(want.shape), (what, got.shape, want.shape)
+    if got.numel() == 0:
+        return
+    viol = float(((got - want).abs() - (ATOL + RTOL * want.abs())).max())
+    assert viol <= 0.0, f"{what}: outside rtol={RTOL} atol={ATOL} by {viol}"
+
+
+def fp64_rows_check(a, b, sizes, trans_b, out, nrows=24, seed=0):
+    """CPU float64 recomputation of a few output rows (first, last and random rows of
+    random experts)."""
+    g = torch.Generator().manual_seed(seed)
+    starts = torch.cumsum(sizes, 0) - sizes
+    for _ in range(nrows):
+        e = int(torch.randint(len(sizes), (1,), generator=g))
+        m = int(sizes[e])
+        if m == 0:
+            continue
+        r = int(starts[e]) + [0, m - 1, int(torch.randint(m, (1,), generator=g))][_ % 3]
+        w = b[e].double().cpu()
+        want = a[r].double().cpu() @ (w.t() if trans_b else w)
+        check(out[r].cpu(), want, f"fp64 row {r} of expert {e}")
+
+
+# ------------------------------------------------ mirrors of the reference's tests
+
+_PROBLEMS = [(z, m, k, n, tb, dev)
+             for (z, m, k, n) in [(1, 128, 128, 128), (8, 128, 128, 128), (16, 128, 128, 128),
+                                  (1, 128, 256, 512), (8, 128, 256, 512), (16, 128, 256, 512)]
+             for tb in (False, True) for dev in (False, True)]          # ops_test.py:20-36
+
+
+def _run_fwd_bwd(ops, oracle, a, b, sizes, trans_b, on_device, legacy_rule=True):
+    bs = sizes.cuda() if on_device else sizes
+    a = a.cuda().requires_grad_(True)
+    b = b.cuda().requires_grad_(True)
+    out = ops.gmm(a, b, bs, trans_b)
+    grad = torch.ones_like(out)                                          # out.sum().backward()
+    out.backward(grad)
+    want, want_ag, want_bg = oracle.gmm_autograd_loop(a.detach().cpu(), b.detach().cpu(), sizes,
+                                                      trans_b, grad.cpu())
+    check(out.detach(), want, "forward")
+    check(a.grad, want_ag, "agrad")
+    check(b.grad, want_bg, "bgrad")
+    if legacy_rule:   # the reference's own acceptance rule, against its own bf16 oracle shape
+        assert oracle.allclose_ops_test(out.detach(), want.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("z,m,k,n,trans_b,on_device", _PROBLEMS)
+def test_fixed_sizes(ops, oracle, z, m, k, n, trans_b, on_device):       # ops_test.py:59-80
+    _announce("fixed", z, m, k, n, trans_b, on_device)
+    torch.manual_seed(0)
+    a = oracle.ops_test_randn(z, m, k).view(-1, k)
+    b = oracle.ops_test_randn(z, n, k) if trans_b else oracle.ops_test_randn(z, k, n)
+    _run_fwd_bwd(ops, oracle, a, b, torch.tensor([m] * z), trans_b, on_device)
+
+
+@pytest.mark.parametrize("z,m,k,n,trans_b,on_device", _PROBLEMS)
+def test_variable_sizes(ops, oracle, z, m, k, n, trans_b, on_device):    # ops_test.py:82-109
+    _announce("variable", z, m, k, n, trans_b, on_device)
+    torch.manual_seed(0)
+    a = oracle.ops_test_randn(z, m, k).view(-1, k)
+    b = oracle.ops_test_randn(z, n, k) if trans_b else oracle.ops_test_randn(z, k, n)
+    dist = torch.rand(z)
+    dist /= dist.sum()
+    sizes = (dist * m).to(torch.long)
+    sizes[-1] += m * z - sizes.sum()
+    assert sizes.sum() == m * z
+    _run_fwd_bwd(ops, oracle, a, b, sizes, trans_b, on_device)
+
+
+@pytest.mark.parametrize("scale", [1.0, 37.0])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_variable_sizes_randn(ops, oracle, trans_b, scale):
+    # same shapes with signed, O(1) data so cancellation and the tolerance are exercised
+    _announce("variable randn", trans_b, scale)
+    g = torch.Generator().manual_seed(1)
+    z, m, k, n = 8, 100, 264, 520
+    sizes = torch.tensor([0, 1, 255, 256, 257, 3, 0, 28])
+    a = (torch.randn(int(sizes.sum()), k, generator=g) * scale).to(torch.bfloat16)
+    b = torch.randn(z, n, k, generator=g).to(torch.bfloat16) if trans_b else \
+        torch.randn(z, k, n, generator=g).to(torch.bfloat16)
+    # tolerance scales with the data: compare after dividing the scale back out
+    bs = sizes
+    out = ops.gmm(a.cuda(), b.cuda(), bs, trans_b)
+    want = oracle.gmm_c(a, b, sizes, trans_b=trans_b)[0]
+    check(out / scale, want / scale, "forward")
+
+
+@pytest.mark.parametrize("on_device", [False, True])
+def test_zero_size_expert_at_mixtral_shape(ops, oracle, on_device):       # ops_test.py:115-141
+    _announce("zero size", on_device)
+    torch.manual_seed(0)
+    m, k, n, e = 16384, 4096, 14336, 8
+    a = oracle.ops_test_randn(e, m // e, k).view(-1, k).cuda().requires_grad_(True)
+    b = oracle.ops_test_randn(e, k, n).cuda().requires_grad_(True)
+    sizes = torch.tensor([219, 2246, 5, 8103, 1, 1117, 4693, 0]).to(torch.long)
+    bs = sizes.cuda() if on_device else sizes
+    out = ops.gmm(a, b, bs)
+    out.sum().backward()
+    ones = torch.ones_like(out)
+    with torch.no_grad():
+        want = oracle.gmm_loop(a.detach(), b.detach(), sizes)                        # fp32, on the GPU
+        want_ag = oracle.gmm_loop(ones, b.detach(), sizes, trans_b=True)
+        want_bg = oracle.gmm_loop(a.detach(), ones, sizes, trans_a=True)
+    check(out.detach(), want, "forward")
+    check(a.grad, want_ag, "agrad")
+    check(b.grad, want_bg, "bgrad")
+    assert (b.grad[7] == 0).all(), "expert without tokens must get a zero weight gradient"
+    fp64_rows_check(a.detach(), b.detach(), sizes, False, out.detach())
+    assert oracle.allclose_ops_test(out.detach(), want.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("on_device", [False, True])
+def test_zero_k_known_answer(ops, on_device):                             # ops_test.py:143-158
+    _announce("zero k", on_device)
+    sz, total = 128, 192
+    a = torch.ones(total, sz).cuda().to(torch.bfloat16)
+    b = torch.ones(total, sz).cuda().to(torch.bfloat16)
+    c = torch.ones(4, sz, sz).cuda().to(torch.bfloat16)
+    bs = torch.tensor([0, 128, 0, 64]).to(torch.long)
+    if on_device:
+        bs = bs.cuda()
+    ret = ops.backend.gmm(a, b, bs, trans_a=True, c=c)
+    assert ret is c
+    assert (c[0] == 0).all() and (c[1] == 128).all() and (c[2] == 0).all() and (c[3] == 64).all()
+
+
+# ------------------------------------------------------ the benchmark configurations
+
+def test_config1_golden_fixture(ops):
+    _announce("config1 fixture")
+    import importlib.util
+    spec = importlib.util.spec_from_file_location(
+        "make_config1", os.path.join(ROOT, "tests", "golden", "make_config1.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    a, b, grad, sizes = mod.inputs()
+    gold = np.load(os.path.join(ROOT, "tests", "golden", "config1.npz"))
+    a = a.cuda().requires_grad_(True)
+    b = b.cuda().requires_grad_(True)
+    out = ops.gmm(a, b, sizes)
+    out.backward(grad.cuda())
+    check(out.detach()[::8], torch.from_numpy(gold["fwd"]), "forward")
+    check(a.grad[::8], torch.from_numpy(gold["agrad"]), "agrad")
+    check(b.grad[:, ::8], torch.from_numpy(gold["bgrad"]), "bgrad")
+
+
+@pytest.mark.parametrize("config,shrink", [(2, 16), (3, 8), (4, 16), (5, 16)])
+@pytest.mark.parametrize("on_device", [False, True])
+def test_configs_shrunk_against_cpu_oracle(ops, oracle, config, shrink, on_device):
+    _announce("config", config, "shrink", shrink, on_device)
+    from grouped_gemm_amd import workloads
+    w = workloads.make(config, device="cuda", shrink=shrink)
+    bs = w.batch_sizes.cuda() if on_device else w.batch_sizes
+    a_cpu, b_cpu, g_cpu = w.a.cpu(), w.b.cpu(), w.grad.cpu()
+    if "fwd" in w.gemms:
+        out = ops.backend.gmm(w.a, w.b, bs, trans_b=w.trans_b)
+        check(out, oracle.gmm_loop(a_cpu, b_cpu, w.batch_sizes, trans_b=w.trans_b), "forward")
+    if "agrad" in w.gemms:
+        ag = ops.backend.gmm(w.grad, w.b, bs, trans_b=not w.trans_b)
+        check(ag, oracle.gmm_loop(g_cpu, b_cpu, w.batch_sizes, trans_b=not w.trans_b), "agrad")
+    if "bgrad" in w.gemms:
+        lhs, rhs = (w.grad, w.a) if w.trans_b else (w.a, w.grad)
+        bg = ops.backend.gmm(lhs, rhs, bs, trans_a=True)
+        want = oracle.gmm_loop(lhs.cpu(), rhs.cpu(), w.batch_sizes, trans_a=True)
+        check(bg, want, "bgrad")
+        empty = (w.batch_sizes == 0).nonzero().flatten().tolist()
+        for e in empty:
+            assert (bg[e] == 0).all()
+
+
+def _full_size_case(ops, oracle, config):
+    from grouped_gemm_amd import workloads
+    w = workloads.make(config, device="cuda")
+    sizes = w.batch_sizes
+    bs = sizes.cuda()
+    results = {}
+    with torch.no_grad():
+        if "fwd" in w.gemms:
+            out = ops.backend.gmm(w.a, w.b, bs, trans_b=w.trans_b)
+            check(out, oracle.gmm_loop(w.a, w.b, sizes, trans_b=w.trans_b), "forward")
+            fp64_rows_check(w.a, w.b, sizes, w.trans_b, out)
+            results["fwd"] = out
+        if "agrad" in w.gemms:
+            ag = ops.backend.gmm(w.grad, w.b, bs, trans_b=not w.trans_b)
+            check(ag, oracle.gmm_loop(w.grad, w.b, sizes, trans_b=not w.trans_b), "agrad")
+            fp64_rows_check(w.grad, w.b, sizes, not w.trans_b, ag, seed=1)
+            del ag
+        if "bgrad" in w.gemms:
+            lhs, rhs = (w.grad, w.a) if w.trans_b else (w.a, w.grad)
+            bg = ops.backend.gmm(lhs, rhs, bs, trans_a=True)
+            starts = torch.cumsum(sizes, 0) - sizes
+            # expert by expert to bound the fp32 copies
+            for e in range(len(sizes)):
+                s, m = int(starts[e]), int(sizes[e])
+                want = lhs[s:s + m].float().t() @ rhs[s:s + m].float()
+                check(bg[e], want, f"bgrad expert {e}")
+            # host-resident sizes must give the very same bits as device-resident ones
+            bg2 = ops.backend.gmm(lhs, rhs, sizes, trans_a=True)
+            assert torch.equal(bg, bg2)
+    return w, results
+
+
+def test_config2_mixtral_full_size(ops, oracle):
+    _announce("config2 full")
+    w, res = _full_size_case(ops, oracle, 2)
+    # linearity in a at full size: gmm(2a, b) == 2 gmm(a, b) bit for bit (power of two)
+    out2 = ops.backend.gmm(w.a * 2, w.b, w.batch_sizes.cuda())
+    assert torch.equal(out2, res["fwd"] * 2)
+
+
+def test_config3_ragged_full_size(ops, oracle):
+    _announce("config3 full")
+    w, res = _full_size_case(ops, oracle, 3)
+    assert int((w.batch_sizes == 0).sum()) >= 4
+    # each expert on its own (one group per call) gives the same bits as the grouped call
+    starts = torch.cumsum(w.batch_sizes, 0) - w.batch_sizes
+    for e in [int(torch.argmax(w.batch_sizes)), int(torch.argmin(w.batch_sizes + (w.batch_sizes == 0) * 10 ** 9))]:
+        s, m = int(starts[e]), int(w.batch_sizes[e])
+        alone = ops.backend.gmm(w.a[s:s + m].contiguous(), w.b[e:e + 1].contiguous(), torch.tensor([m]))
+        assert torch.equal(alone, res["fwd"][s:s + m])
+
+
+def test_config4_weight_gradient_full_size(ops, oracle):
+    _announce("config4 full")
+    _full_size_case(ops, oracle, 4)
+
+
+def test_config5_deepseek_share_full_size_autograd(ops, oracle):
+    _announce("config5 full")
+    from grouped_gemm_amd import workloads
+    w = workloads.make(5, device="cuda")
+    sizes = w.batch_sizes
+    a = w.a.requires_grad_(True)
+    b = w.b.requires_grad_(True)
+    out = ops.gmm(a, b, sizes.cuda(), True)
+    out.backward(w.grad)
+    with torch.no_grad():
+        check(out.detach(), oracle.gmm_loop(w.a.detach(), w.b.detach(), sizes, trans_b=True), "forward")
+        check(a.grad, oracle.gmm_loop(w.grad, w.b.detach(), sizes, trans_b=False), "agrad")
+        starts = torch.cumsum(sizes, 0) - sizes
+        for e in range(len(sizes)):
+            s, m = int(starts[e]), int(sizes[e])
+            want = w.grad[s:s + m].float().t() @ w.a.detach()[s:s + m].float()
+            check(b.grad[e], want, f"bgrad expert {e}")
+        fp64_rows_check(w.a.detach(), w.b.detach(), sizes, True, out.detach())
+
+
+# ----------------------------------------------------------------- schedule, bit-exact
+
+SCHED_CASES = [
+    ([128] * 8, 128, 128),
+    ([219, 2246, 5, 8103, 1, 1117, 4693, 0], 4096, 14336),
+    ([0, 0, 0], 64, 64),
+    ([256] * 256, 7168, 2048),          # b offsets pass 2**31 elements
+    ([1] * 512, 8, 8),
+    ([70000, 0, 3, 70000], 2048, 1408),
+]
+
+
+@pytest.mark.parametrize("sizes,hin,hout", SCHED_CASES)
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+@pytest.mark.parametrize("on_device", [False, True])
+def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
+    trans_a, trans_b = layout
+    _announce("schedule", len(sizes), hin, hout, layout, on_device)
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    tokens = int(bs.sum())
+    got = ops.backend.debug_schedule(bs.cuda() if on_device else bs, tokens, hin, hout, trans_a, trans_b).cpu().numpy()
+    want = oracle.table_closed(sizes, hin, hout, trans_a, trans_b)
+    assert np.array_equal(got[:, :9], want)
+    assert np.array_equal(want, oracle.table_walk(sizes, hin, hout, trans_a, trans_b)[0])
+    # tiles: consecutive, non-overlapping, and enough to cover each group's output
+    assert np.array_equal(got[:, 9], np.cumsum(got[:, 10]) - got[:, 10])
+    assert np.array_equal(got[:, 11], np.array(sizes))
+    lib = ctypes.CDLL(os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so"))
+    bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    lib.gg_tile_shape(int(trans_a), int(trans_b), ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk))
+    m, n = got[:, 0], got[:, 1]
+    assert np.array_equal(got[:, 10], -(-m // bm.value) * -(-n // bn.value))
+
+
+def test_schedule_clips_rows_past_tokens(ops):
+    # device-resident sizes that claim more rows than `a` has: clipped, never followed
+    bs = torch.tensor([100, 100, 100], dtype=torch.int64).cuda()
+    got = ops.backend.debug_schedule(bs, 150, 64, 64, False, False).cpu().numpy()
+    assert got[:, 11].tolist() == [100, 50, 0]
+    assert got[:, 6].tolist() == [0, 100 * 64, 150 * 64]
+
+
+# ----------------------------------------------------------------- C ABI, directly
+
+def _c_abi():
+    lib = ctypes.CDLL(os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so"))
+    lib.gg_last_error.restype = ctypes.c_char_p
+    lib.gg_gmm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    return lib
+
+
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+@pytest.mark.parametrize("on_device", [False, True])
+def test_c_abi_against_c_oracle(oracle, layout, on_device):
+    trans_a, trans_b = layout
+    _announce("c abi", layout, on_device)
+    lib = _c_abi()
+    g = torch.Generator().manual_seed(7)
+    sizes = torch.tensor([5, 0, 300, 64, 1, 0, 130], dtype=torch.int64)
+    t, hin, hout = int(sizes.sum()), 72, 264
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    if trans_a:
+        b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+        c = torch.full((len(sizes), hin, hout), 7.0, dtype=torch.bfloat16)
+    else:
+        b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+        c = torch.full((t, hout), 7.0, dtype=torch.bfloat16)
+    da, db, dc = a.cuda(), b.cuda(), c.cuda()
+    dsz = sizes.cuda() if on_device else sizes
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        rc = lib.gg_gmm_bf16(da.data_ptr(), db.data_ptr(), dc.data_ptr(), dsz.data_ptr(), int(on_device),
+                             len(sizes), t, hin, hout, int(trans_a), int(trans_b), stream.cuda_stream)
+    assert rc == 0, lib.gg_last_error()
+    stream.synchronize()
+    want32, _ = oracle.gmm_c(a, b, sizes, trans_a=trans_a, trans_b=trans_b)
+    check(dc, want32, "c abi")
+    if trans_a:
+        assert (dc[1] == 0).all() and (dc[5] == 0).all()
+
+
+def test_c_abi_rejects_bad_host_sizes():
+    lib = _c_abi()
+    a = torch.zeros(16, 8, dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros(2, 8, 8, dtype=torch.bfloat16, device="cuda")
+    c = torch.zeros(16, 8, dtype=torch.bfloat16, device="cuda")
+    for sizes in ([10, 10], [-1, 4]):
+        s = torch.tensor(sizes, dtype=torch.int64)
+        rc = lib.gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), s.data_ptr(), 0, 2, 16, 8, 8, 0, 0, None)
+        assert rc == -1, sizes
+    s = torch.zeros(513, dtype=torch.int64, device="cuda")
+    rc = lib.gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), s.data_ptr(), 1, 513, 16, 8, 8, 0, 0, None)
+    assert rc == -2 and b"512" in lib.gg_last_error()
+
+
+# ------------------------------------------------------------------------ edge cases
+
+def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):
+    g = torch.Generator().manual_seed(3)
+    sizes = torch.tensor([40, 0, 300])
+    a = torch.randn(400, 64, generator=g).to(torch.bfloat16).cuda()     # 60 rows past the groups
+    b = torch.randn(3, 64, 72, generator=g).to(torch.bfloat16).cuda()
+    c = torch.full((400, 72), float("nan"), dtype=torch.bfloat16, device="cuda")
+    ops.backend.gmm(a, b, sizes, c=c)
+    assert not torch.isnan(c[:340]).any()
+    assert torch.isnan(c[340:]).all()
+    check(c[:340], oracle.gmm_loop(a.cpu(), b.cpu(), sizes)[:340], "forward")
+
+
+def test_all_experts_empty(ops):
+    a = torch.zeros(0, 64, dtype=torch.bfloat16, device="cuda")
+    b = torch.randn(4, 64, 72, device="cuda").to(torch.bfloat16)
+    sizes = torch.zeros(4, dtype=torch.int64)
+    out = ops.backend.gmm(a, b, sizes)
+    assert out.shape == (0, 72)
+    c = torch.ones(4, 64, 72, dtype=torch.bfloat16, device="cuda")
+    ops.backend.gmm(a, torch.zeros(0, 72, dtype=torch.bfloat16, device="cuda"), sizes.cuda(), trans_a=True, c=c)
+    assert (c == 0).all()
+
+
+def test_more_than_512_experts(ops, oracle):
+    g = torch.Generator().manual_seed(5)
+    e = 700
+    sizes = torch.randint(0, 6, (e,), generator=g)
+    t = int(sizes.sum())
+    a = torch.randn(t, 32, generator=g).to(torch.bfloat16)
+    b = torch.randn(e, 32, 40, generator=g).to(torch.bfloat16)
+    out = ops.backend.gmm(a.cuda(), b.cuda(), sizes)                      # host sizes: split launches
+    check(out, oracle.gmm_loop(a, b, sizes), "forward")
+    grad = torch.randn(t, 40, generator=g).to(torch.bfloat16)
+    bg = ops.backend.gmm(a.cuda(), grad.cuda(), sizes, trans_a=True)
+    check(bg, oracle.gmm_loop(a, grad, sizes, trans_a=True), "bgrad")
+    with pytest.raises(RuntimeError, match="512"):                       # csrc/grouped_gemm.cu:120-124
+        ops.backend.gmm(a.cuda(), b.cuda(), sizes.cuda())
+
+
+def test_gpu_validation_errors(ops):
+    a = torch.zeros(8, 16, dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros(2, 16, 24, dtype=torch.bfloat16, device="cuda")
+    bs = torch.tensor([3, 5])
+    with pytest.raises(RuntimeError):
+        ops.backend.gmm(a, b.cpu(), bs)
+    with pytest.raises(RuntimeError):
+        ops.backend.gmm(a, b, bs.int())
+    with pytest.raises(RuntimeError):
+        ops.backend.gmm(a, b, torch.tensor([3, 6]))                       # sums past the rows of a
+    with pytest.raises(RuntimeError):
+        ops.backend.gmm(a, b, bs, c=torch.zeros(8, 32, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        ops.backend.gmm(a[:, :12].contiguous(), b[:, :12].contiguous(), bs)
+    with pytest.raises(AssertionError):
+        ops.backend.gmm(a, b, bs, trans_a=True, trans_b=True)
+
+
+def test_needs_input_grad_is_respected(ops):
+    a = torch.randn(64, 32, device="cuda").to(torch.bfloat16).requires_grad_(True)
+    b = torch.randn(2, 32, 40, device="cuda").to(torch.bfloat16)
+    out = ops.gmm(a, b, torch.tensor([30, 34]))
+    out.sum().backward()
+    assert a.grad is not None and b.grad is None
+
+
+def test_runs_on_the_current_stream(ops, oracle):
+    g = torch.Generator().manual_seed(11)
+    sizes = torch.tensor([500, 12])
+    a = torch.randn(512, 256, generator=g).to(torch.bfloat16).cuda()
+    b = torch.randn(2, 256, 128, generator=g).to(torch.bfloat16).cuda()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        a2 = a * 2          # produced on s; the kernel must be ordered after it on s
+        out = ops.backend.gmm(a2, b, sizes.cuda())
+    s.synchronize()
+    check(out / 2, oracle.gmm_loop(a.cpu(), b.cpu(), sizes), "forward")

@@ -1,0 +1,185 @@
+"""CPU-only checks of the host side: the Python surface mirrors the reference's, every
+validation rule raises before the device is touched, the C-ABI library loads and
+exports what include/grouped_gemm_hip.h declares, and the golden fixture of
+configuration 1 still matches the oracle.  No GPU, no compute calls."""
+import ctypes
+import importlib.util
+import inspect
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HIP_LIB = os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so")
+
+
+def bf16(*shape):
+    return torch.zeros(*shape, dtype=torch.bfloat16)
+
+
+# ------------------------------------------------------------------ Python surface
+
+def test_package_layout_matches_reference():
+    # grouped_gemm/__init__.py:1-2, ops.py:1, ops_test.py:5,154
+    import grouped_gemm
+    from grouped_gemm import ops
+    import grouped_gemm.backend as be
+    import grouped_gemm_backend
+    assert ops.backend is be
+    assert be.backend is grouped_gemm_backend
+    assert list(inspect.signature(ops.gmm).parameters) == ["a", "b", "batch_sizes", "trans_b"]
+    assert list(inspect.signature(be.gmm).parameters) == ["a", "b", "batch_sizes", "trans_a", "trans_b", "c"]
+    assert inspect.signature(be.gmm).parameters["c"].default is None
+    assert issubclass(ops.GroupedGemm, torch.autograd.Function)
+
+
+def test_allocate_output_shapes_and_asserts():
+    # grouped_gemm/backend.py:11-22
+    from grouped_gemm_amd.backend import _allocate_output
+    bs = torch.tensor([3, 5])
+    assert _allocate_output(bf16(8, 16), bf16(2, 16, 24), bs, False, False).shape == (8, 24)
+    assert _allocate_output(bf16(8, 16), bf16(2, 24, 16), bs, False, True).shape == (8, 24)
+    out = _allocate_output(bf16(8, 16), bf16(8, 24), bs, True, False)
+    assert out.shape == (2, 16, 24) and out.dtype == torch.bfloat16
+    with pytest.raises(AssertionError):
+        _allocate_output(bf16(8, 16), bf16(8, 24), bs, True, True)
+    with pytest.raises(AssertionError):
+        _allocate_output(bf16(8, 16), bf16(2, 16, 24), bs.view(1, 2), False, False)
+    with pytest.raises(AssertionError):
+        _allocate_output(bf16(2, 4, 16), bf16(2, 16, 24), bs, False, False)
+    with pytest.raises(AssertionError):
+        _allocate_output(bf16(8, 16), bf16(16, 24), bs, False, False)
+    with pytest.raises(AssertionError):
+        _allocate_output(bf16(8, 16), bf16(2, 8, 24), bs, True, False)
+
+
+def test_cpu_tensors_are_rejected_by_gmm():
+    # csrc/grouped_gemm.cu:490: a must be on the GPU; surfaces as RuntimeError
+    from grouped_gemm import ops
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ops.gmm(bf16(8, 16), bf16(2, 16, 24), torch.tensor([3, 5]))
+
+
+GOOD = dict(a=(8, 16), b=(2, 16, 24), c=(8, 24), bs=[3, 5], ta=False, tb=False)
+
+
+def _validate(**kw):
+    import grouped_gemm_backend
+    cfg = dict(GOOD)
+    cfg.update(kw)
+    a = cfg.get("a_t", bf16(*cfg["a"]))
+    b = cfg.get("b_t", bf16(*cfg["b"]))
+    c = cfg.get("c_t", bf16(*cfg["c"]))
+    bs = cfg.get("bs_t", torch.tensor(cfg["bs"], dtype=torch.int64))
+    grouped_gemm_backend.validate(a, b, c, bs, cfg["ta"], cfg["tb"])
+
+
+def test_validate_accepts_the_three_layouts():
+    _validate()
+    _validate(b=(2, 24, 16), tb=True)
+    _validate(b=(8, 24), c=(2, 16, 24), ta=True)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(ta=True, tb=True),                                     # grouped_gemm.cu:476
+    dict(bs_t=torch.tensor([[3, 5]])),                          # :485
+    dict(bs_t=torch.tensor([3, 5], dtype=torch.int32)),         # :486
+    dict(a=(2, 4, 16)),                                         # :491
+    dict(a_t=torch.zeros(8, 16)),                               # :492
+    dict(b_t=torch.zeros(2, 16, 24, dtype=torch.float16)),      # :505
+    dict(c_t=torch.zeros(8, 24)),                               # :506
+    dict(ta=True, b=(2, 4, 24), c=(2, 16, 24)),                 # :517
+    dict(ta=True, b=(8, 24), c=(2 * 16, 24)),                   # :518
+    dict(ta=True, b=(7, 24), c=(2, 16, 24)),                    # :519
+    dict(ta=True, b=(8, 24), c=(3, 16, 24)),                    # :520
+    dict(ta=True, b=(8, 24), c=(2, 8, 24)),                     # :521
+    dict(ta=True, b=(8, 24), c=(2, 16, 32)),                    # :522
+    dict(b=(16, 24)),                                           # :524
+    dict(c=(2, 4, 24)),                                         # :525
+    dict(b=(2, 8, 24)),                                         # :531 contraction mismatch
+    dict(tb=True),                                              # :531 with trans_b: b.size(2) != a.size(1)
+    dict(bs=[3, 4, 1]),                                         # :534
+    dict(c=(8, 32)),                                            # output shape (checked here, not in the reference)
+    dict(a_t=bf16(16, 8).t()),                                  # :538
+    dict(b_t=bf16(2, 24, 16).transpose(1, 2)),                  # :539
+    dict(c_t=bf16(24, 8).t()),                                  # :540
+])
+def test_validate_rejects(kw):
+    with pytest.raises(RuntimeError):
+        _validate(**kw)
+
+
+# ------------------------------------------------------------------------ C ABI
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "grouped_gemm_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert {"gg_gmm_bf16", "gg_debug_schedule", "gg_last_error", "gg_version", "gg_tile_shape"} <= set(names)
+    lib = ctypes.CDLL(HIP_LIB)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_c_abi_argument_errors_need_no_device():
+    lib = ctypes.CDLL(HIP_LIB)
+    lib.gg_last_error.restype = ctypes.c_char_p
+    i64 = ctypes.c_int64
+    sizes = (i64 * 2)(3, 5)
+    call = lambda hin, hout, ta, tb, tokens=8, e=2: lib.gg_gmm_bf16(
+        None, None, None, sizes, 0, i64(e), i64(tokens), i64(hin), i64(hout), ta, tb, None)
+    assert call(16, 24, 1, 1) == -1 and b"both" in lib.gg_last_error()
+    assert call(16, 20, 0, 0) == -2 and b"multiples of 8" in lib.gg_last_error()
+    assert call(-8, 24, 0, 0) == -1
+    assert call(16, 24, 0, 0, tokens=1 << 31) == -2
+    assert call(16, 24, 0, 0, e=0) == 0                       # nothing to do
+    bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert lib.gg_tile_shape(0, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
+    assert bm.value > 0 and bn.value > 0 and bk.value > 0
+    assert lib.gg_version() >= 100
+
+
+# ----------------------------------------------------------------- workloads
+
+def test_workload_generators():
+    from grouped_gemm_amd import workloads
+    g = torch.Generator().manual_seed(0)
+    s2 = workloads.router_sizes(16384, 8, 2, g)
+    assert int(s2.sum()) == 32768 and s2.numel() == 8 and int(s2.min()) > 0
+    s3 = workloads.zipf_sizes(49152, 64, 1.2, 4, g)
+    assert int(s3.sum()) == 49152 and int((s3 == 0).sum()) >= 4
+    s5 = workloads.poisson_sizes(65536, 256, g)
+    assert int(s5.sum()) == 65536 and s5.numel() == 256 and int(s5.min()) >= 0
+    w = workloads.make(3, device="cpu", shrink=16)
+    assert w.a.shape == (49152 // 16, 128) and w.b.shape == (64, 128, 88) and not w.trans_b
+    assert int(w.batch_sizes.sum()) == w.tokens
+    w5 = workloads.make(5, device="cpu", shrink=32)
+    assert w5.trans_b and w5.b.shape == (256, 64, 224)
+    assert w5.flops_per_gemm() == 2 * w5.tokens * 224 * 64
+
+
+# -------------------------------------------------------------- golden fixture
+
+def test_config1_fixture_matches_oracle(oracle):
+    spec = importlib.util.spec_from_file_location(
+        "make_config1", os.path.join(ROOT, "tests", "golden", "make_config1.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    a, b, grad, sizes = mod.inputs()
+    fwd, agrad, bgrad = mod.expected(a, b, grad, sizes)
+    gold = np.load(os.path.join(ROOT, "tests", "golden", "config1.npz"))
+    assert np.array_equal(gold["fwd"], fwd[::8].numpy())
+    assert np.array_equal(gold["agrad"], agrad[::8].numpy())
+    assert np.array_equal(gold["bgrad"], bgrad[:, ::8].numpy())
+    # the same numbers from the library routine, by autograd through the loop
+    out, ag, bg = oracle.gmm_autograd_loop(a, b, sizes, False, grad)
+    torch.testing.assert_close(out, fwd, rtol=1e-5, atol=1e-4)
+    torch.testing.assert_close(ag, agrad, rtol=1e-5, atol=1e-4)
+    torch.testing.assert_close(bg, bgrad, rtol=1e-5, atol=1e-4)
