@@ -175,12 +175,11 @@ struct GroupGeom {
   int32_t m, n, k;
 };
 
+// `start` and `rows` are the group's entries of Sched::row_start and Sched::rows.
 template <int LAYOUT>
-__device__ __forceinline__ GroupGeom group_geometry(const Sched* s, const GmmParams& p, int e) {
+__device__ __forceinline__ GroupGeom group_geometry(const GmmParams& p, int e, int64_t start,
+                                                    int rows) {
   GroupGeom g;
-  // read through the first lane: everything derived from these stays in scalar registers
-  const int64_t start = uniform(s->row_start[e]);
-  const int rows = uniform(s->rows[e]);
   const int64_t hin = p.hidden_in, hout = p.hidden_out;
   if (LAYOUT == kTN) {
     g.m = p.hidden_in;
@@ -221,7 +220,7 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(
   build_schedule<LAYOUT, BM, BN, HOST_SIZES>(&s, p, hs);
   __syncthreads();
   for (int e = threadIdx.x; e < p.num_groups; e += 64) {
-    const GroupGeom g = group_geometry<LAYOUT>(&s, p, e);
+    const GroupGeom g = group_geometry<LAYOUT>(p, e, s.row_start[e], s.rows[e]);
     int64_t* row = p.sched_out + (int64_t)e * kSchedCols;
     row[0] = g.m;
     row[1] = g.n;
@@ -458,7 +457,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   int e = 0;
   for (int t = vid; t < total_tiles; t += G) {
     while (t >= uniform(sched->tile_start[e + 1])) ++e;
-    const GroupGeom g = group_geometry<LAYOUT>(sched, p, e);
+    // read through the first lane: everything derived from these stays in scalar registers
+    const GroupGeom g = group_geometry<LAYOUT>(p, e, uniform(sched->row_start[e]),
+                                               uniform(sched->rows[e]));
     const int u = t - uniform(sched->tile_start[e]);
     const int tiles_m = LAYOUT == kTN ? tiles_m_fixed : (g.m + BM - 1) / BM;
     int tm, tn;

@@ -307,7 +307,7 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
     tokens = int(bs.sum())
     got = ops.backend.debug_schedule(bs.cuda() if on_device else bs, tokens, hin, hout, trans_a, trans_b).cpu().numpy()
     want = oracle.table_closed(sizes, hin, hout, trans_a, trans_b)
-    assert np.array_equal(got[:, :9], want)
+    np.testing.assert_array_equal(got[:, :9], want)
     assert np.array_equal(want, oracle.table_walk(sizes, hin, hout, trans_a, trans_b)[0])
     # tiles: consecutive, non-overlapping, and enough to cover each group's output
     assert np.array_equal(got[:, 9], np.cumsum(got[:, 10]) - got[:, 10])
