@@ -19,7 +19,7 @@ HIP_LIB = os.path.join(HERE, "libgrouped_gemm_hip.so")
 EXT_LIB = os.path.join(HERE, "grouped_gemm_backend" + sysconfig.get_config_var("EXT_SUFFIX"))
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-shared",
     # packed fp32 instructions are switched off for device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",

@@ -30,8 +30,24 @@ int fail(int code, const char* fmt, ...) {
       return fail(GG_EHIP, "%s failed: %s", #call, hipGetErrorString(err__));            \
   } while (0)
 
-// Tile configuration per layout.
-constexpr int BM = 256, BN = 256, BK = 64, STAGES = 2, WAVES_M = 2, WAVES_N = 2;
+// Tile configuration (build-time tunables; the defaults are what ships).
+#ifndef GG_BK
+#define GG_BK 64
+#endif
+#ifndef GG_STAGES
+#define GG_STAGES 2
+#endif
+#ifndef GG_GROUP_M
+#define GG_GROUP_M 4
+#endif
+#ifndef GG_WAVES_M
+#define GG_WAVES_M 2
+#endif
+#ifndef GG_WAVES_N
+#define GG_WAVES_N 2
+#endif
+constexpr int BM = 256, BN = 256, BK = GG_BK, STAGES = GG_STAGES;
+constexpr int WAVES_M = GG_WAVES_M, WAVES_N = GG_WAVES_N;
 constexpr int kThreads = WAVES_M * WAVES_N * 64;
 
 struct DeviceInfo {
@@ -166,7 +182,7 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
   p.tokens = tokens;
   p.hidden_in = (int32_t)hidden_in;
   p.hidden_out = (int32_t)hidden_out;
-  p.group_m = 8;
+  p.group_m = GG_GROUP_M;
   p.sched_out = nullptr;
 
   if (batch_sizes_on_device) {
@@ -250,7 +266,7 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   p.tokens = tokens;
   p.hidden_in = (int32_t)hidden_in;
   p.hidden_out = (int32_t)hidden_out;
-  p.group_m = 8;
+  p.group_m = GG_GROUP_M;
   p.num_groups = (int32_t)num_groups;
   p.sched_out = table_out;
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);

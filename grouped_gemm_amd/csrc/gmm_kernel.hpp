@@ -19,6 +19,7 @@
 #include <stdint.h>
 
 #include <type_traits>
+#include <utility>
 
 namespace gg {
 
@@ -66,14 +67,46 @@ constexpr uint32_t kRsrcFlags = 0x00020000u;   // raw buffer, 32-bit data format
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// Descriptor of `bytes` bytes at `base`.  Both are the same in every lane; reading them
-// through the first lane tells the compiler so and keeps the descriptor in scalar registers.
+// Buffer descriptor of `bytes` bytes at `base`, as the four dwords the hardware reads.
+// Both inputs are the same in every lane; reading them through the first lane tells the
+// compiler so and keeps the descriptor in scalar registers.
+using rsrc_words = __attribute__((ext_vector_type(4))) int;
+
+__device__ __forceinline__ rsrc_words make_rsrc_words(const void* base, uint32_t bytes) {
+  const uint64_t b = reinterpret_cast<uint64_t>(base);
+  rsrc_words r;
+  r[0] = uniform((int)(uint32_t)b);
+  r[1] = uniform((int)((uint32_t)(b >> 32) & 0xffffu));   // 48-bit base, stride 0
+  r[2] = uniform((int)bytes);
+  r[3] = (int)kRsrcFlags;
+  return r;
+}
+
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   const uint64_t b = reinterpret_cast<uint64_t>(base);
   const uint64_t ub = (uint64_t)(uint32_t)uniform((int)(uint32_t)b) |
                       ((uint64_t)(uint32_t)uniform((int)(uint32_t)(b >> 32)) << 32);
   return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(ub), 0,
                                            (uint32_t)uniform((int)bytes), kRsrcFlags);
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_addr + lane * 16.
+// Written as assembly on purpose: the compiler then keeps no record of pending writes
+// into LDS, and does not put a full wait for them in front of later LDS reads that touch
+// other buffers of the ring.  The waits that are needed are the explicit wait_vmcnt calls.
+__device__ __forceinline__ void load_to_lds_16(const rsrc_words& rsrc, uint32_t voffset,
+                                               uint32_t lds_addr) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %0, %1, 0 offen lds"
+      :
+      : "v"(voffset), "s"(rsrc), "s"(lds_addr)
+      : "memory");
+}
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)reinterpret_cast<uintptr_t>(GG_LDS_PTR(p));
 }
 
 template <int N>
@@ -266,7 +299,7 @@ struct DepthMajor {
 
   const char* base;   // first row of the tile, depth 0
   int ld;             // elements between rows ( = depth extent )
-  int rows_valid;     // rows of the tile that exist
+  int span;           // elements from the tile's first row to its last existing row
   int depth;          // depth extent
   int my_chunk;       // depth chunk (of 8) this lane fetches
   uint32_t voff0;     // byte offset of this lane's chunk for load 0
@@ -274,7 +307,7 @@ struct DepthMajor {
   __device__ __forceinline__ void setup(const char* tile_base, int ld_, int rows_valid_, int depth_) {
     base = tile_base;
     ld = ld_;
-    rows_valid = rows_valid_;
+    span = rows_valid_ > 0 ? (rows_valid_ - 1) * ld_ : -(1 << 30);   // no rows: nothing in range
     depth = depth_;
     const int tid = threadIdx.x;
     const int row = tid / CPR, pos = tid % CPR;
@@ -283,20 +316,24 @@ struct DepthMajor {
   }
 
   // Fetch depth slice [kt*BK, kt*BK+BK) into the LDS tile at `dst` (wave-uniform).
-  __device__ __forceinline__ void issue(int kt, char* dst, int wave) const {
+  // What all loads of depth slice kt share.
+  struct Slice {
+    rsrc_words rsrc;
+    uint32_t v0;   // this lane's offset for load 0, or out of range in the depth tail
+  };
+  __device__ __forceinline__ Slice slice(int kt) const {
     const int left = uniform(depth - kt * BK);
-    const uint32_t bytes = (left > 0 && rows_valid > 0)
-                               ? (uint32_t)((rows_valid - 1) * ld + left) * 2u : 0u;
-    const __amdgpu_buffer_rsrc_t r = make_rsrc(base + (int64_t)kt * (BK * 2), bytes);
-    uint32_t v = voff0;
-    if (left < BK) v = (my_chunk * 8 < left) ? v : kOutOfRange;   // depth tail, uniform branch
+    const int elems = left > 0 ? span + left : 0;
+    Slice sl;
+    sl.rsrc = make_rsrc_words(base + (int64_t)kt * (BK * 2), elems > 0 ? (uint32_t)elems * 2u : 0u);
+    sl.v0 = (left >= BK || my_chunk * 8 < left) ? voff0 : kOutOfRange;
+    return sl;
+  }
+  // Load I of the NI that make up one slice, into the LDS tile at `dst` (wave-uniform).
+  template <int I>
+  __device__ __forceinline__ void load(const Slice& sl, const char* dst, int wave) const {
     const uint32_t step = (uint32_t)(ROWS_PER_INSTR * ld) * 2u;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, GG_LDS_PTR(dst + (i * NT + wave * 64) * 16), 16,
-                                               v, 0, 0, 0);
-      v += step;
-    }
+    load_to_lds_16(sl.rsrc, sl.v0 + I * step, uniform(lds_address(dst) + (I * NT + wave * 64) * 16));
   }
 };
 
@@ -336,16 +373,19 @@ struct WidthMajor {
     }
   }
 
-  __device__ __forceinline__ void issue(int kt, char* dst, int wave) const {
+  struct Slice {
+    rsrc_words rsrc;
+  };
+  __device__ __forceinline__ Slice slice(int kt) const {
     int left = uniform(depth - kt * BK);
     left = left < 0 ? 0 : (left > BK ? BK : left);
-    const __amdgpu_buffer_rsrc_t r =
-        make_rsrc(base + (int64_t)kt * BK * ld * 2, (uint32_t)(left * ld) * 2u);
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, GG_LDS_PTR(dst + (i * NT + wave * 64) * 16), 16,
-                                               voff[i], 0, 0, 0);
-    }
+    Slice sl;
+    sl.rsrc = make_rsrc_words(base + (int64_t)kt * BK * ld * 2, (uint32_t)(left * ld) * 2u);
+    return sl;
+  }
+  template <int I>
+  __device__ __forceinline__ void load(const Slice& sl, const char* dst, int wave) const {
+    load_to_lds_16(sl.rsrc, voff[I], uniform(lds_address(dst) + (I * NT + wave * 64) * 16));
   }
 };
 
@@ -402,6 +442,14 @@ struct WidthMajorFrag {
 
 // ------------------------------------------------------------------------ kernel
 
+// Compile-time loop: f(integral_constant<int, 0>{}), ..., f(integral_constant<int, N-1>{}).
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  [&]<int... I>(std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+  }(std::make_integer_sequence<int, N>{});
+}
+
 template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N>
 struct GmmConfig {
   static constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -416,18 +464,71 @@ struct GmmConfig {
   static_assert(BK % 16 == 0 && STAGES >= 2, "");
 };
 
+// One output tile as the scheduler hands it out.
+struct TileInfo {
+  GroupGeom g;
+  int m0, n0;       // first row and column of the tile inside its group's output
+  int rows_valid;   // rows of the tile that exist (0: no tile)
+  int nk;           // depth slices, at least 1 so that an empty group still stores zeros
+  bool valid;
+};
+
+// Tile index -> group and position.  `e` is the caller's cursor into the groups; tile
+// indices only grow, so it only moves forward.
+template <int LAYOUT, int BM, int BN, int BK>
+__device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParams& p, int t,
+                                              int total_tiles, int& e) {
+  TileInfo ti;
+  if (t >= total_tiles) {
+    ti.g = GroupGeom{0, 0, 0, 0, 0, 0};
+    ti.m0 = ti.n0 = ti.rows_valid = 0;
+    ti.nk = 1;
+    ti.valid = false;
+    return ti;
+  }
+  while (t >= uniform(sched->tile_start[e + 1])) ++e;
+  // read through the first lane: everything derived from these stays in scalar registers
+  ti.g = group_geometry<LAYOUT>(p, e, uniform(sched->row_start[e]), uniform(sched->rows[e]));
+  const int u = t - uniform(sched->tile_start[e]);
+  const int tiles_n = (ti.g.n + BN - 1) / BN;
+  const int tiles_m = (ti.g.m + BM - 1) / BM;
+  int tm, tn;
+  tile_coords(u, tiles_m, tiles_n, p.group_m, &tm, &tn);
+  ti.m0 = uniform(tm) * BM;
+  ti.n0 = uniform(tn) * BN;
+  ti.rows_valid = min(BM, ti.g.m - ti.m0);
+  const int nk = (ti.g.k + BK - 1) / BK;
+  ti.nk = nk < 1 ? 1 : nk;
+  ti.valid = true;
+  return ti;
+}
+
 template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool HOST_SIZES>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     GmmParams p, std::conditional_t<HOST_SIZES, HostSizes, NoSizes> hs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
-  constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB;
+  constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB, KS = BK / 16;
   using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT>, WidthMajor<BM, BK, NT>>;
   using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT>, WidthMajor<BN, BK, NT>>;
   using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BM, BK, MB>>;
   using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BN, BK, NB>>;
-  constexpr int LOADS_PER_TILE = ALoad::NI + BLoad::NI;
-  static_assert((STAGES - 2) * LOADS_PER_TILE < 64, "too many loads in flight for vmcnt");
+  constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;
+  // With three or more buffers the loads of a slice are issued in KS parts, one per 16-deep
+  // step, so that the memory pipe sees a steady trickle instead of a burst that would hold
+  // up the MFMAs queued behind it.  With two buffers the slice is issued at once.
+  constexpr bool SPREAD = STAGES >= 3;
+  constexpr int PARTS = SPREAD ? KS : 1;
+  static_assert(ALoad::NI % PARTS == 0 || PARTS % 2 == 0, "");
+  constexpr int PART_LOADS = LOADS_PER_STAGE / PARTS;
+  static_assert(LOADS_PER_STAGE % PARTS == 0 && (ALoad::NI % PART_LOADS == 0 || PART_LOADS % ALoad::NI == 0),
+                "a part holds loads of one operand, or whole operands");
+  constexpr int IN_FLIGHT = (STAGES - 2) * LOADS_PER_STAGE;   // loads allowed to be pending
+  constexpr int PROLOGUE_IN_FLIGHT = SPREAD ? IN_FLIGHT + PART_LOADS : (STAGES - 1) * LOADS_PER_STAGE;
+  static_assert(PROLOGUE_IN_FLIGHT < 64, "too many loads in flight for vmcnt");
+  static_assert(KS % 2 == 0, "the two fragment sets alternate per 16-deep step");
+  constexpr int UNITS = MB + NB;    // fragments read per 16-deep step
+  constexpr int SLOTS = MB * NB;    // MFMAs per 16-deep step
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   Sched* sched = reinterpret_cast<Sched*>(smem + STAGES * Cfg::STAGE_BYTES);
@@ -443,100 +544,156 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   afrag.setup(wm * Cfg::WTM);
   bfrag.setup(wn * Cfg::WTN);
 
-  const int E = p.num_groups;
-  const int total_tiles = uniform(sched->tile_start[E]);
-  const int tiles_n = (p.hidden_out + BN - 1) / BN;
-  const int tiles_m_fixed = (p.hidden_in + BM - 1) / BM;   // TN only
+  const int total_tiles = uniform(sched->tile_start[p.num_groups]);
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
   // tile indices so that its private L2 sees neighbouring tiles.
   const int G = gridDim.x;
   const int w = blockIdx.x;
   const int vid = (G % 8 == 0) ? (w % 8) * (G / 8) + (w / 8) : w;
+  if (vid >= total_tiles) return;
 
-  int e = 0;
-  for (int t = vid; t < total_tiles; t += G) {
-    while (t >= uniform(sched->tile_start[e + 1])) ++e;
-    // read through the first lane: everything derived from these stays in scalar registers
-    const GroupGeom g = group_geometry<LAYOUT>(p, e, uniform(sched->row_start[e]),
-                                               uniform(sched->rows[e]));
-    const int u = t - uniform(sched->tile_start[e]);
-    const int tiles_m = LAYOUT == kTN ? tiles_m_fixed : (g.m + BM - 1) / BM;
-    int tm, tn;
-    tile_coords(u, tiles_m, tiles_n, p.group_m, &tm, &tn);
-    tm = uniform(tm);
-    tn = uniform(tn);
-    const int m0 = tm * BM, n0 = tn * BN;
-    const int rows_valid = min(BM, g.m - m0);
-    const int depth = g.k;
-    const int nk = (depth + BK - 1) / BK;
-
-    ALoad aload;
-    BLoad bload;
+  // Two cursors walk this workgroup's tiles: the fetch cursor runs STAGES depth slices
+  // ahead of the compute cursor and crosses into the next tile on its own, so the first
+  // slices of a tile are already in flight while the previous tile is being stored.
+  ALoad aload;
+  BLoad bload;
+  int fetch_t = vid, fetch_e = 0, fetch_kt = 0;
+  TileInfo fti;
+  auto fetch_setup = [&]() {
+    fti = find_tile<LAYOUT, BM, BN, BK>(sched, p, fetch_t, total_tiles, fetch_e);
+    const int depth = fti.valid ? fti.g.k : 0;
     if constexpr (Cfg::A_DEPTH_MAJOR) {
-      aload.setup(p.a + (g.a_off + (int64_t)m0 * g.k) * 2, g.k, rows_valid, depth);
+      aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * 2, fti.g.k, fti.rows_valid, depth);
     } else {
-      aload.setup(p.a + g.a_off * 2, g.m, depth, m0, g.m);
+      aload.setup(p.a + fti.g.a_off * 2, fti.g.m, depth, fti.m0, fti.g.m);
     }
     if constexpr (Cfg::B_DEPTH_MAJOR) {
-      bload.setup(p.b + (g.b_off + (int64_t)n0 * g.k) * 2, g.k, min(BN, g.n - n0), depth);
+      bload.setup(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
+                  fti.valid ? min(BN, fti.g.n - fti.n0) : 0, depth);
     } else {
-      bload.setup(p.b + g.b_off * 2, g.n, depth, n0, g.n);
+      bload.setup(p.b + fti.g.b_off * 2, fti.g.n, depth, fti.n0, fti.g.n);
     }
+  };
+  // Slices past the depth (or past the last tile) are fetched with an empty descriptor:
+  // zeros, no traffic, and the number of loads in flight is the same at every step.
+  typename ALoad::Slice a_slice;
+  typename BLoad::Slice b_slice;
+  auto fetch_begin = [&]() {   // descriptors of the cursor's slice
+    a_slice = aload.slice(fetch_kt);
+    b_slice = bload.slice(fetch_kt);
+  };
+  // Load J of the cursor's slice (A's loads first, then B's) into buffer `buf`.
+  auto fetch_load = [&](auto j_tag, int buf) {
+    constexpr int J = decltype(j_tag)::value;
+    const char* st = smem + buf * Cfg::STAGE_BYTES;
+    if constexpr (J < ALoad::NI) {
+      aload.template load<J>(a_slice, st, wave);
+    } else {
+      bload.template load<J - ALoad::NI>(b_slice, st + Cfg::A_BYTES, wave);
+    }
+  };
+  auto fetch_advance = [&]() {
+    if (++fetch_kt == fti.nk && fti.valid) {
+      fetch_t += G;
+      fetch_kt = 0;
+      fetch_setup();
+    }
+  };
 
-    f32x16 acc[MB][NB];
+  // Fragments: two register sets that alternate per 16-deep step.  A "unit" is one
+  // fragment (one ds_read_b128, or two transposing 64-bit reads): A's MB first, then B's NB.
+  bf16x8 fa[2][MB], fb[2][NB];
+  auto read_unit = [&](auto u_tag, auto set_tag, int buf, int ks) {
+    constexpr int U = decltype(u_tag)::value, SET = decltype(set_tag)::value;
+    const char* sa = smem + buf * Cfg::STAGE_BYTES;
+    if constexpr (U < MB) {
+      fa[SET][U] = afrag.read(sa, ks, U);
+    } else {
+      fb[SET][U - MB] = bfrag.read(sa + Cfg::A_BYTES, ks, U - MB);
+    }
+  };
+
+  f32x16 acc[MB][NB];
+  auto zero_acc = [&]() {
 #pragma unroll
     for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int j = 0; j < NB; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  };
 
-    // every wave is done reading the previous tile's buffers
-    block_barrier();
+  fetch_setup();
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) {
-      char* st = smem + s * Cfg::STAGE_BYTES;
-      aload.issue(s, st, wave);
-      bload.issue(s, st + Cfg::A_BYTES, wave);
+  for (int s = 0; s < (SPREAD ? STAGES - 1 : STAGES); ++s) {
+    fetch_begin();
+    static_for<LOADS_PER_STAGE>([&](auto j) { fetch_load(j, s); });
+    fetch_advance();
+  }
+  if constexpr (SPREAD) {
+    fetch_begin();
+    static_for<PART_LOADS>([&](auto j) { fetch_load(j, STAGES - 1); });
+  }
+
+  int tile_t = vid, tile_e = 0;
+  TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, total_tiles, tile_e);
+  wait_vmcnt<PROLOGUE_IN_FLIGHT>();   // the first slice is in
+  block_barrier();
+  static_for<UNITS>([&](auto u) { read_unit(u, std::integral_constant<int, 0>{}, 0, 0); });
+
+  int rd = 0;
+  int fill = STAGES - 1;   // buffer the fetch cursor is filling
+  while (true) {
+    zero_acc();
+    for (int kt = 0; kt < ti.nk; ++kt) {
+      static_for<KS>([&](auto ks_tag) {
+        constexpr int ks = decltype(ks_tag)::value;
+        constexpr int cur = ks & 1, nxt = cur ^ 1;
+        constexpr bool last = ks + 1 == KS;
+        // which loads of the cursor's slice go out in this step
+        constexpr int first_load = SPREAD ? (last ? 0 : (ks + 1) * PART_LOADS) : 0;
+        constexpr int num_loads = SPREAD ? PART_LOADS : (last ? LOADS_PER_STAGE : 0);
+        int src = rd;   // buffer the next fragments come from
+        if constexpr (last) {
+          // The next slice has landed for every wave, and every wave holds its fragments of
+          // this slice in registers: this slice's buffer is free for the slice STAGES ahead.
+          wait_vmcnt<IN_FLIGHT>();
+          block_barrier();
+          fill = rd;
+          fetch_begin();
+          rd = rd + 1 == STAGES ? 0 : rd + 1;
+          src = rd;
+        }
+        // The step as SLOTS slots of one MFMA each; the LDS reads of the next step's
+        // fragments and this step's share of global loads go out behind the first MFMAs, in
+        // this order, so they run under the matrix pipe.
+        static_for<SLOTS>([&](auto m_tag) {
+          constexpr int m = decltype(m_tag)::value;
+          constexpr int i = m / NB, j = m % NB;
+          // operands swapped: the result block is held transposed, so a lane owns four
+          // consecutive columns of one output row
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+          constexpr int u0 = UNITS * m / SLOTS, u1 = UNITS * (m + 1) / SLOTS;
+          static_for<u1 - u0>([&](auto d) {
+            read_unit(std::integral_constant<int, u0 + decltype(d)::value>{},
+                      std::integral_constant<int, nxt>{}, src, last ? 0 : ks + 1);
+          });
+          constexpr int l0 = num_loads * m / SLOTS, l1 = num_loads * (m + 1) / SLOTS;
+          static_for<l1 - l0>([&](auto d) {
+            fetch_load(std::integral_constant<int, first_load + l0 + decltype(d)::value>{}, fill);
+          });
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        // the cursor moves on once the last load of its slice is out
+        if constexpr (SPREAD ? (ks + 2 == KS) : last) fetch_advance();
+      });
     }
-    int rd = 0, wr = STAGES - 1;
-    for (int kt = 0; kt < nk; ++kt) {
-      wait_vmcnt<(STAGES - 2) * LOADS_PER_TILE>();
-      block_barrier();
-      {
-        // slices past the depth are fetched with an empty descriptor: zeros, no traffic,
-        // and the count of loads in flight stays the same in every iteration
-        char* st = smem + wr * Cfg::STAGE_BYTES;
-        aload.issue(kt + STAGES - 1, st, wave);
-        bload.issue(kt + STAGES - 1, st + Cfg::A_BYTES, wave);
-      }
-      const char* sa = smem + rd * Cfg::STAGE_BYTES;
-      const char* sb = sa + Cfg::A_BYTES;
-#pragma unroll
-      for (int ks = 0; ks < BK / 16; ++ks) {
-        bf16x8 af[MB], bfv[NB];
-#pragma unroll
-        for (int i = 0; i < MB; ++i) af[i] = afrag.read(sa, ks, i);
-#pragma unroll
-        for (int j = 0; j < NB; ++j) bfv[j] = bfrag.read(sb, ks, j);
-#pragma unroll
-        for (int i = 0; i < MB; ++i)
-#pragma unroll
-          for (int j = 0; j < NB; ++j)
-            // operands swapped: the result block is held transposed, so a lane owns four
-            // consecutive columns of one output row
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfv[j], af[i], acc[i][j], 0, 0, 0);
-      }
-      rd = rd + 1 == STAGES ? 0 : rd + 1;
-      wr = wr + 1 == STAGES ? 0 : wr + 1;
-    }
-    wait_vmcnt<0>();
 
     // epilogue: lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3
     {
-      const char* cbase = p.c + (g.c_off + (int64_t)m0 * g.n) * 2;
-      const uint32_t cbytes = rows_valid > 0 ? (uint32_t)(rows_valid * g.n) * 2u : 0u;
+      const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * 2;
+      const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * 2u : 0u;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
 #pragma unroll
       for (int i = 0; i < MB; ++i) {
@@ -545,17 +702,30 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
         for (int j = 0; j < NB; ++j) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const int col = n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+            const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+            // The accumulators stay in the accumulation registers; each value is moved out
+            // right where it is converted, so the epilogue needs only a few vector registers.
             bf16x4 o;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[i][j][4 * q + r];
-            const uint32_t off = col < g.n ? (uint32_t)(row * g.n + col) * 2u : kOutOfRange;
+            for (int r = 0; r < 4; ++r) {
+              float v;
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
+              o[r] = (__bf16)v;
+            }
+            const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
             __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, o), rc, off, 0, 0);
           }
+          // keep the conversion of one block from being hoisted over the stores of the
+          // previous one: at most 16 accumulators are live in vector registers at a time
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
+    tile_t += G;
+    if (tile_t >= total_tiles) break;
+    ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, total_tiles, tile_e);
   }
+  wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
