@@ -513,20 +513,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT>, WidthMajor<BN, BK, NT>>;
   using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BM, BK, MB>>;
   using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BN, BK, NB>>;
-  constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;
-  // With three or more buffers the loads of a slice are issued in KS parts, one per 16-deep
-  // step, so that the memory pipe sees a steady trickle instead of a burst that would hold
-  // up the MFMAs queued behind it.  With two buffers the slice is issued at once.
-  constexpr bool SPREAD = STAGES >= 3;
-  constexpr int PARTS = SPREAD ? KS : 1;
-  static_assert(ALoad::NI % PARTS == 0 || PARTS % 2 == 0, "");
-  constexpr int PART_LOADS = LOADS_PER_STAGE / PARTS;
-  static_assert(LOADS_PER_STAGE % PARTS == 0 && (ALoad::NI % PART_LOADS == 0 || PART_LOADS % ALoad::NI == 0),
-                "a part holds loads of one operand, or whole operands");
-  constexpr int IN_FLIGHT = (STAGES - 2) * LOADS_PER_STAGE;   // loads allowed to be pending
-  constexpr int PROLOGUE_IN_FLIGHT = SPREAD ? IN_FLIGHT + PART_LOADS : (STAGES - 1) * LOADS_PER_STAGE;
-  static_assert(PROLOGUE_IN_FLIGHT < 64, "too many loads in flight for vmcnt");
-  static_assert(KS % 2 == 0, "the two fragment sets alternate per 16-deep step");
+  constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;   // per lane, per depth slice
+  constexpr int HALF_LOADS = LOADS_PER_STAGE / 2;
+  static_assert(KS == 4 && STAGES == 2, "the step schedule below is written for BK = 64 and two buffers");
+  static_assert(LOADS_PER_STAGE % 2 == 0 && LOADS_PER_STAGE < 32, "");
   constexpr int UNITS = MB + NB;    // fragments read per 16-deep step
   constexpr int SLOTS = MB * NB;    // MFMAs per 16-deep step
 
@@ -601,16 +591,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     }
   };
 
-  // Fragments: two register sets that alternate per 16-deep step.  A "unit" is one
-  // fragment (one ds_read_b128, or two transposing 64-bit reads): A's MB first, then B's NB.
-  bf16x8 fa[2][MB], fb[2][NB];
-  auto read_unit = [&](auto u_tag, auto set_tag, int buf, int ks) {
+  // Fragments: one register set per 16-deep step of a slice.  A "unit" is one fragment (one
+  // ds_read_b128, or two transposing 64-bit reads): A's MB first, then B's NB.
+  bf16x8 fa[KS][MB], fb[KS][NB];
+  auto read_unit = [&](auto u_tag, auto set_tag, int buf) {   // set = 16-deep step it belongs to
     constexpr int U = decltype(u_tag)::value, SET = decltype(set_tag)::value;
     const char* sa = smem + buf * Cfg::STAGE_BYTES;
     if constexpr (U < MB) {
-      fa[SET][U] = afrag.read(sa, ks, U);
+      fa[SET][U] = afrag.read(sa, SET, U);
     } else {
-      fb[SET][U - MB] = bfrag.read(sa + Cfg::A_BYTES, ks, U - MB);
+      fb[SET][U - MB] = bfrag.read(sa + Cfg::A_BYTES, SET, U - MB);
     }
   };
 
@@ -624,70 +614,82 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
   };
 
+  // One 16-deep step: SLOTS slots of one MFMA each, with this step's LDS reads and global
+  // loads placed behind the first MFMAs, in this order, so they run under the matrix pipe.
+  //   READS   fragments to fetch: unit u < UNITS goes to set READ_SET, units beyond to READ_SET+1
+  //   LOADS   global loads FIRST_LOAD .. of the fetch cursor's slice, into buffer `fill`
+  auto step = [&](auto ks_tag, auto reads_tag, auto read_set_tag, auto first_load_tag,
+                  auto loads_tag, int src, int fill) {
+    constexpr int ks = decltype(ks_tag)::value, READS = decltype(reads_tag)::value;
+    constexpr int READ_SET = decltype(read_set_tag)::value;
+    constexpr int FIRST_LOAD = decltype(first_load_tag)::value, LOADS = decltype(loads_tag)::value;
+    static_for<SLOTS>([&](auto m_tag) {
+      constexpr int m = decltype(m_tag)::value;
+      constexpr int i = m / NB, j = m % NB;
+      // operands swapped: the result block is held transposed, so a lane owns four
+      // consecutive columns of one output row
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+      constexpr int u0 = READS * m / SLOTS, u1 = READS * (m + 1) / SLOTS;
+      static_for<u1 - u0>([&](auto d) {
+        constexpr int u = u0 + decltype(d)::value;
+        read_unit(std::integral_constant<int, u % UNITS>{},
+                  std::integral_constant<int, READ_SET + u / UNITS>{}, src);
+      });
+      constexpr int l0 = LOADS * m / SLOTS, l1 = LOADS * (m + 1) / SLOTS;
+      static_for<l1 - l0>([&](auto d) {
+        fetch_load(std::integral_constant<int, FIRST_LOAD + l0 + decltype(d)::value>{}, fill);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using IU = std::integral_constant<int, UNITS>;
+  using IU2 = std::integral_constant<int, 2 * UNITS>;
+  using IH = std::integral_constant<int, HALF_LOADS>;
+
   fetch_setup();
 #pragma unroll
-  for (int s = 0; s < (SPREAD ? STAGES - 1 : STAGES); ++s) {
+  for (int s = 0; s < 2; ++s) {
     fetch_begin();
     static_for<LOADS_PER_STAGE>([&](auto j) { fetch_load(j, s); });
     fetch_advance();
   }
-  if constexpr (SPREAD) {
-    fetch_begin();
-    static_for<PART_LOADS>([&](auto j) { fetch_load(j, STAGES - 1); });
-  }
 
   int tile_t = vid, tile_e = 0;
   TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, total_tiles, tile_e);
-  wait_vmcnt<PROLOGUE_IN_FLIGHT>();   // the first slice is in
+  wait_vmcnt<LOADS_PER_STAGE>();   // the first slice is in
   block_barrier();
-  static_for<UNITS>([&](auto u) { read_unit(u, std::integral_constant<int, 0>{}, 0, 0); });
+  static_for<2 * UNITS>([&](auto u) {
+    constexpr int uu = decltype(u)::value;
+    read_unit(std::integral_constant<int, uu % UNITS>{}, std::integral_constant<int, uu / UNITS>{}, 0);
+  });
 
-  int rd = 0;
-  int fill = STAGES - 1;   // buffer the fetch cursor is filling
+  // Per slice: steps 0 and 1 read the fragments of steps 2 and 3 from the slice's buffer X.
+  // After that nobody needs X any more: a barrier at step 2 hands it to the fetch cursor, which
+  // fills it with the slice two ahead during steps 2 and 3.  The other buffer Y must be
+  // complete only at step 3, where the first two steps' fragments of the next slice are read.
+  // Releasing X one step before Y is needed keeps loads in flight across the hand-over.
+  int x = 0;   // buffer of the slice being multiplied
   while (true) {
     zero_acc();
     for (int kt = 0; kt < ti.nk; ++kt) {
-      static_for<KS>([&](auto ks_tag) {
-        constexpr int ks = decltype(ks_tag)::value;
-        constexpr int cur = ks & 1, nxt = cur ^ 1;
-        constexpr bool last = ks + 1 == KS;
-        // which loads of the cursor's slice go out in this step
-        constexpr int first_load = SPREAD ? (last ? 0 : (ks + 1) * PART_LOADS) : 0;
-        constexpr int num_loads = SPREAD ? PART_LOADS : (last ? LOADS_PER_STAGE : 0);
-        int src = rd;   // buffer the next fragments come from
-        if constexpr (last) {
-          // The next slice has landed for every wave, and every wave holds its fragments of
-          // this slice in registers: this slice's buffer is free for the slice STAGES ahead.
-          wait_vmcnt<IN_FLIGHT>();
-          block_barrier();
-          fill = rd;
-          fetch_begin();
-          rd = rd + 1 == STAGES ? 0 : rd + 1;
-          src = rd;
-        }
-        // The step as SLOTS slots of one MFMA each; the LDS reads of the next step's
-        // fragments and this step's share of global loads go out behind the first MFMAs, in
-        // this order, so they run under the matrix pipe.
-        static_for<SLOTS>([&](auto m_tag) {
-          constexpr int m = decltype(m_tag)::value;
-          constexpr int i = m / NB, j = m % NB;
-          // operands swapped: the result block is held transposed, so a lane owns four
-          // consecutive columns of one output row
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
-          constexpr int u0 = UNITS * m / SLOTS, u1 = UNITS * (m + 1) / SLOTS;
-          static_for<u1 - u0>([&](auto d) {
-            read_unit(std::integral_constant<int, u0 + decltype(d)::value>{},
-                      std::integral_constant<int, nxt>{}, src, last ? 0 : ks + 1);
-          });
-          constexpr int l0 = num_loads * m / SLOTS, l1 = num_loads * (m + 1) / SLOTS;
-          static_for<l1 - l0>([&](auto d) {
-            fetch_load(std::integral_constant<int, first_load + l0 + decltype(d)::value>{}, fill);
-          });
-          __builtin_amdgcn_sched_barrier(0);
-        });
-        // the cursor moves on once the last load of its slice is out
-        if constexpr (SPREAD ? (ks + 2 == KS) : last) fetch_advance();
-      });
+      const int y = x ^ 1;
+      step(I0{}, IU{}, I2{}, I0{}, I0{}, x, x);
+      step(I1{}, IU{}, I3{}, I0{}, I0{}, x, x);
+      // every wave has all fragments of this slice in registers
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      block_barrier();
+      fetch_begin();
+      step(I2{}, I0{}, I0{}, I0{}, IH{}, x, x);
+      // the next slice has landed for every wave (only the loads just issued may be pending)
+      wait_vmcnt<HALF_LOADS>();
+      block_barrier();
+      step(I3{}, IU2{}, I0{}, IH{}, IH{}, y, x);
+      fetch_advance();
+      x = y;
     }
 
     // epilogue: lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3
