@@ -514,9 +514,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BM, BK, MB>>;
   using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BN, BK, NB>>;
   constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;   // per lane, per depth slice
-  constexpr int HALF_LOADS = LOADS_PER_STAGE / 2;
+  constexpr int QUARTER_LOADS = LOADS_PER_STAGE / 4;
   static_assert(KS == 4 && STAGES == 2, "the step schedule below is written for BK = 64 and two buffers");
-  static_assert(LOADS_PER_STAGE % 2 == 0 && LOADS_PER_STAGE < 32, "");
+  static_assert(LOADS_PER_STAGE % 4 == 0 && LOADS_PER_STAGE < 32, "");
   constexpr int UNITS = MB + NB;    // fragments read per 16-deep step
   constexpr int SLOTS = MB * NB;    // MFMAs per 16-deep step
 
@@ -646,49 +646,55 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  using IU = std::integral_constant<int, UNITS>;
   using IU2 = std::integral_constant<int, 2 * UNITS>;
-  using IH = std::integral_constant<int, HALF_LOADS>;
+  using IQ = std::integral_constant<int, QUARTER_LOADS>;
+  using IQ2 = std::integral_constant<int, 2 * QUARTER_LOADS>;
+  using IQ3 = std::integral_constant<int, 3 * QUARTER_LOADS>;
 
+  // Both buffers are requested up front, except the last quarter of the second slice: every
+  // step issues one quarter of a slice's loads, and step 0 issues the last quarter of the
+  // slice that was begun in the steps before it.
   fetch_setup();
-#pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    fetch_begin();
-    static_for<LOADS_PER_STAGE>([&](auto j) { fetch_load(j, s); });
-    fetch_advance();
-  }
+  fetch_begin();
+  static_for<LOADS_PER_STAGE>([&](auto j) { fetch_load(j, 0); });
+  fetch_advance();
+  fetch_begin();
+  static_for<3 * QUARTER_LOADS>([&](auto j) { fetch_load(j, 1); });
 
   int tile_t = vid, tile_e = 0;
   TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, total_tiles, tile_e);
-  wait_vmcnt<LOADS_PER_STAGE>();   // the first slice is in
+  wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
     constexpr int uu = decltype(u)::value;
     read_unit(std::integral_constant<int, uu % UNITS>{}, std::integral_constant<int, uu / UNITS>{}, 0);
   });
 
-  // Per slice: steps 0 and 1 read the fragments of steps 2 and 3 from the slice's buffer X.
-  // After that nobody needs X any more: a barrier at step 2 hands it to the fetch cursor, which
-  // fills it with the slice two ahead during steps 2 and 3.  The other buffer Y must be
-  // complete only at step 3, where the first two steps' fragments of the next slice are read.
-  // Releasing X one step before Y is needed keeps loads in flight across the hand-over.
+  // Per slice (buffer X, the other buffer Y holds the next slice):
+  //   step 0  reads the fragments of steps 2 and 3 from X; after it nobody needs X any more
+  //   step 1  barrier: X goes to the fetch cursor, which starts the slice two ahead into it
+  //   step 3  barrier: Y is complete for every wave; reads the fragments of the next slice's
+  //           steps 0 and 1 from Y
+  // Every step issues a quarter of a slice's loads (step 0 the last quarter of the slice begun
+  // in steps 1-3 before it), so the memory pipe sees a steady trickle, and X is released two
+  // steps before Y is needed, so loads stay in flight across the hand-over.
   int x = 0;   // buffer of the slice being multiplied
   while (true) {
     zero_acc();
     for (int kt = 0; kt < ti.nk; ++kt) {
       const int y = x ^ 1;
-      step(I0{}, IU{}, I2{}, I0{}, I0{}, x, x);
-      step(I1{}, IU{}, I3{}, I0{}, I0{}, x, x);
+      step(I0{}, IU2{}, I2{}, IQ3{}, IQ{}, x, y);
+      fetch_advance();
       // every wave has all fragments of this slice in registers
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       block_barrier();
       fetch_begin();
-      step(I2{}, I0{}, I0{}, I0{}, IH{}, x, x);
-      // the next slice has landed for every wave (only the loads just issued may be pending)
-      wait_vmcnt<HALF_LOADS>();
+      step(I1{}, I0{}, I0{}, I0{}, IQ{}, x, x);
+      step(I2{}, I0{}, I0{}, IQ{}, IQ{}, x, x);
+      // the next slice has landed for every wave (only this slice's two quarters may be pending)
+      wait_vmcnt<2 * QUARTER_LOADS>();
       block_barrier();
-      step(I3{}, IU2{}, I0{}, IH{}, IH{}, y, x);
-      fetch_advance();
+      step(I3{}, IU2{}, I0{}, IQ2{}, IQ{}, y, x);
       x = y;
     }
 
