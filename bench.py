@@ -27,6 +27,14 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2516.6   # 256 CU x 4096 flop/clk x 2.4 GHz, dense
 PEAK_HBM_GBPS = 8000.0
 
+# Bytes per launch between L2 and the fabric for the default workload, from two rocprofv3 --pmc
+# runs of this file (FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by a 1 GiB device copy, both in
+# KiB); the figures and commands are in profiles/gmm_kernel_mixtral_w1_hbm_traffic.md.
+MEASURED_TRAFFIC_BYTES = {
+    2: {"fwd": (3180011 * 2.0 + 917830) * 1024, "agrad": (3279799 * 2.0 + 262174) * 1024,
+        "bgrad": (2753398 * 2.0 + 917708) * 1024},
+}
+
 
 def cpu_baseline(w, budget_s=12.0):
     """Oracle loop on the host cores: forward, input gradient and weight gradient of the
@@ -78,6 +86,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration (2 = Mixtral w1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zeros", action="store_true",
+                    help="diagnostic: all-zero inputs (no data toggling), to separate the power "
+                         "limit from the kernel's cycle efficiency; not a valid benchmark result")
+    ap.add_argument("--copy-bytes", type=int, default=0,
+                    help="only run a plain device copy of this many bytes, 5 times (a known "
+                         "traffic to scale the FETCH_SIZE / WRITE_SIZE counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; expert-parallel sharding across GPUs "
@@ -89,7 +103,17 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
+    if args.copy_bytes:
+        src = torch.ones(args.copy_bytes, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copied_bytes": args.copy_bytes, "times": 5}))
+        return
     w = workloads.make(args.config, device="cuda")
+    if args.zeros:
+        w.a.zero_(), w.b.zero_(), w.grad.zero_()
     sizes_dev = w.batch_sizes.cuda()
     lhs, rhs = (w.grad, w.a) if w.trans_b else (w.a, w.grad)
     calls = {
@@ -142,7 +166,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic",
+        "data": "zeros (diagnostic, not a benchmark result)" if args.zeros else "synthetic",
         "config": {
             "workload": f"configs[{args.config - 1}]: {w.batch_sizes.numel()} experts, {w.tokens} routed rows, "
                         f"{w.hidden_in}x{w.hidden_out}, forward + input-gradient + weight-gradient grouped GEMMs",
@@ -157,7 +181,9 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": (round(MEASURED_TRAFFIC_BYTES[args.config][slowest])
+                        if args.config in MEASURED_TRAFFIC_BYTES and not args.zeros else None),
+            "algorithmic_bytes": bytes_gemm,
             "launch_ms": round(kernel_ms[slowest], 4),
             "flops_per_launch": flops_gemm,
             "per_kernel": {
