@@ -33,6 +33,7 @@ using bf16x4 = __attribute__((ext_vector_type(4))) __bf16;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 using f32x4 = __attribute__((ext_vector_type(4))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) uint32_t;
+using u32x4 = __attribute__((ext_vector_type(4))) uint32_t;
 
 #define GG_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
@@ -459,7 +460,16 @@ struct GmmConfig {
   static constexpr bool B_DEPTH_MAJOR = LAYOUT == kNT;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LDS_BYTES = STAGES * STAGE_BYTES + (int)sizeof(Sched);
+  // after the tile buffers: the schedule, then one strip per wave for the epilogue
+  static constexpr int SCHED_OFFSET = STAGES * STAGE_BYTES;
+  static constexpr int EPILOGUE_OFFSET = (SCHED_OFFSET + (int)sizeof(Sched) + 15) / 16 * 16;
+  static constexpr int EPILOGUE_PITCH = 64 * 2 + 16;            // 64 bf16 columns + padding
+  static constexpr int EPILOGUE_WAVE_BYTES = 32 * EPILOGUE_PITCH;
+  static constexpr bool STAGED_EPILOGUE =
+      NB % 2 == 0 && EPILOGUE_OFFSET + WAVES_M * WAVES_N * EPILOGUE_WAVE_BYTES <= 160 * 1024;
+  static constexpr int LDS_BYTES =
+      STAGED_EPILOGUE ? EPILOGUE_OFFSET + WAVES_M * WAVES_N * EPILOGUE_WAVE_BYTES
+                      : SCHED_OFFSET + (int)sizeof(Sched);
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
   static_assert(BK % 16 == 0 && STAGES >= 2, "");
 };
@@ -521,7 +531,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   constexpr int SLOTS = MB * NB;    // MFMAs per 16-deep step
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  Sched* sched = reinterpret_cast<Sched*>(smem + STAGES * Cfg::STAGE_BYTES);
+  Sched* sched = reinterpret_cast<Sched*>(smem + Cfg::SCHED_OFFSET);
   build_schedule<LAYOUT, BM, BN, HOST_SIZES>(sched, p, hs);
   __syncthreads();
 
@@ -698,34 +708,68 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
       x = y;
     }
 
-    // epilogue: lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3
+    // Epilogue.  A lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3.
+    // The accumulators stay in the accumulation registers; each value is moved out right
+    // where it is converted, so the epilogue needs only a few vector registers.
     {
       const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * 2;
       const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * 2u : 0u;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
+      auto take4 = [&](int i, int j, int q) {
+        bf16x4 o;
 #pragma unroll
-      for (int i = 0; i < MB; ++i) {
-        const int row = wm * Cfg::WTM + i * 32 + (lane & 31);
+        for (int r = 0; r < 4; ++r) {
+          float v;
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
+          o[r] = (__bf16)v;
+        }
+        return __builtin_bit_cast(u32x2, o);
+      };
+      if constexpr (Cfg::STAGED_EPILOGUE) {
+        // Through a strip of LDS private to the wave: 32 rows x 64 columns go in as the
+        // 8-byte pieces the lanes hold and come out as 16 bytes per lane, 8 lanes per row, so
+        // that one store instruction writes 8 complete 128-byte lines.
+        char* strip = smem + Cfg::EPILOGUE_OFFSET + wave * Cfg::EPILOGUE_WAVE_BYTES;
+        constexpr int PITCH = Cfg::EPILOGUE_PITCH;
+        const int in_row = lane & 31, in_half = lane >> 5;
+        const int out_row = lane >> 3, out_chunk = lane & 7;
 #pragma unroll
-        for (int j = 0; j < NB; ++j) {
+        for (int i = 0; i < MB; ++i) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
-            // The accumulators stay in the accumulation registers; each value is moved out
-            // right where it is converted, so the epilogue needs only a few vector registers.
-            bf16x4 o;
+          for (int jp = 0; jp < NB / 2; ++jp) {
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<u32x2*>(strip + in_row * PITCH + (jj * 32 + 8 * q + 4 * in_half) * 2) =
+                    take4(i, 2 * jp + jj, q);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              float v;
-              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
-              o[r] = (__bf16)v;
+              const u32x4 v = *reinterpret_cast<const u32x4*>(strip + (r * 8 + out_row) * PITCH + out_chunk * 16);
+              const int row = wm * Cfg::WTM + i * 32 + r * 8 + out_row;
+              const int col = ti.n0 + wn * Cfg::WTN + jp * 64 + out_chunk * 8;
+              const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
+              __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, 0);
             }
-            const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, o), rc, off, 0, 0);
+            // keep the conversion of one strip from being hoisted over the stores of the
+            // previous one: few accumulators are live in vector registers at a time
+            __builtin_amdgcn_sched_barrier(0);
           }
-          // keep the conversion of one block from being hoisted over the stores of the
-          // previous one: at most 16 accumulators are live in vector registers at a time
-          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+          const int row = wm * Cfg::WTM + i * 32 + (lane & 31);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+              const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
+              __builtin_amdgcn_raw_buffer_store_b64(take4(i, j, q), rc, off, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       }
     }
