@@ -30,25 +30,27 @@ int fail(int code, const char* fmt, ...) {
       return fail(GG_EHIP, "%s failed: %s", #call, hipGetErrorString(err__));            \
   } while (0)
 
-// Tile configuration (build-time tunables; the defaults are what ships).
-#ifndef GG_BK
-#define GG_BK 64
-#endif
-#ifndef GG_STAGES
-#define GG_STAGES 2
-#endif
+// Tile shapes.  Wide: 256 x 256 outputs per workgroup, 2 x 2 waves of 128 x 128.  Short: 128 x 256,
+// 1 x 4 waves of 128 x 64, for calls whose groups have few rows (a group of 257 rows costs two
+// 256-row tiles but barely more than two 128-row ones).  The weight-gradient layout always
+// uses the wide shape: its ragged dimension is the depth, not the rows.
 #ifndef GG_GROUP_M
 #define GG_GROUP_M 4
 #endif
-#ifndef GG_WAVES_M
-#define GG_WAVES_M 2
+#ifndef GG_SHORT_BELOW
+#define GG_SHORT_BELOW 112   // average rows per group below which the short shape is used
 #endif
-#ifndef GG_WAVES_N
-#define GG_WAVES_N 2
-#endif
-constexpr int BM = 256, BN = 256, BK = GG_BK, STAGES = GG_STAGES;
-constexpr int WAVES_M = GG_WAVES_M, WAVES_N = GG_WAVES_N;
-constexpr int kThreads = WAVES_M * WAVES_N * 64;
+constexpr int BK = 64, STAGES = 2;
+struct Wide {
+  static constexpr int BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2;
+};
+struct Short {
+  static constexpr int BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
+};
+
+bool use_short_shape(int64_t num_groups, int64_t tokens, int trans_a) {
+  return !trans_a && num_groups > 0 && tokens < (int64_t)GG_SHORT_BELOW * num_groups;
+}
 
 struct DeviceInfo {
   int cus = 0;
@@ -74,11 +76,12 @@ int device_info(DeviceInfo* out) {
   return GG_OK;
 }
 
-template <int LAYOUT, bool HOST_SIZES>
+template <typename S, int LAYOUT, bool HOST_SIZES>
 int launch(const gg::GmmParams& p, const gg::HostSizes* hs, int grid, hipStream_t stream) {
-  using Cfg = gg::GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
+  using Cfg = gg::GmmConfig<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N>;
+  constexpr int kThreads = S::WAVES_M * S::WAVES_N * 64;
   const void* kernel = reinterpret_cast<const void*>(
-      &gg::gmm_kernel<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N, HOST_SIZES>);
+      &gg::gmm_kernel<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, HOST_SIZES>);
   // raising the dynamic LDS limit is per device and per kernel; do it once each
   static std::mutex mu;
   static bool done[64] = {};
@@ -107,9 +110,9 @@ int launch(const gg::GmmParams& p, const gg::HostSizes* hs, int grid, hipStream_
   return GG_OK;
 }
 
-template <int LAYOUT, bool HOST_SIZES>
+template <typename S, int LAYOUT, bool HOST_SIZES>
 int launch_dump(const gg::GmmParams& p, const gg::HostSizes* hs, hipStream_t stream) {
-  auto kernel = gg::schedule_dump_kernel<LAYOUT, BM, BN, HOST_SIZES>;
+  auto kernel = gg::schedule_dump_kernel<LAYOUT, S::BM, S::BN, HOST_SIZES>;
   if constexpr (HOST_SIZES) {
     hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, stream, p, *hs);
   } else {
@@ -117,6 +120,30 @@ int launch_dump(const gg::GmmParams& p, const gg::HostSizes* hs, hipStream_t str
   }
   GG_HIP(hipGetLastError());
   return GG_OK;
+}
+
+template <bool HOST_SIZES>
+int dispatch(bool short_shape, int layout, const gg::GmmParams& p, const gg::HostSizes* hs, int grid,
+             hipStream_t stream) {
+  if (layout == gg::kTN) return launch<Wide, gg::kTN, HOST_SIZES>(p, hs, grid, stream);
+  if (short_shape) {
+    return layout == gg::kNN ? launch<Short, gg::kNN, HOST_SIZES>(p, hs, grid, stream)
+                             : launch<Short, gg::kNT, HOST_SIZES>(p, hs, grid, stream);
+  }
+  return layout == gg::kNN ? launch<Wide, gg::kNN, HOST_SIZES>(p, hs, grid, stream)
+                           : launch<Wide, gg::kNT, HOST_SIZES>(p, hs, grid, stream);
+}
+
+template <bool HOST_SIZES>
+int dispatch_dump(bool short_shape, int layout, const gg::GmmParams& p, const gg::HostSizes* hs,
+                  hipStream_t stream) {
+  if (layout == gg::kTN) return launch_dump<Wide, gg::kTN, HOST_SIZES>(p, hs, stream);
+  if (short_shape) {
+    return layout == gg::kNN ? launch_dump<Short, gg::kNN, HOST_SIZES>(p, hs, stream)
+                             : launch_dump<Short, gg::kNT, HOST_SIZES>(p, hs, stream);
+  }
+  return layout == gg::kNN ? launch_dump<Wide, gg::kNN, HOST_SIZES>(p, hs, stream)
+                           : launch_dump<Wide, gg::kNT, HOST_SIZES>(p, hs, stream);
 }
 
 int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens, int64_t hidden_in,
@@ -136,10 +163,10 @@ int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens,
 
 // Upper bound of the tile count for any size vector (the device clips rows to `tokens`).
 int64_t tile_bound(int64_t num_groups, int64_t tokens, int64_t hidden_in, int64_t hidden_out,
-                   int trans_a) {
-  const int64_t tiles_n = (hidden_out + BN - 1) / BN;
-  if (trans_a) return num_groups * ((hidden_in + BM - 1) / BM) * tiles_n;
-  return (tokens / BM + num_groups) * tiles_n;
+                   int trans_a, int bm, int bn) {
+  const int64_t tiles_n = (hidden_out + bn - 1) / bn;
+  if (trans_a) return num_groups * ((hidden_in + bm - 1) / bm) * tiles_n;
+  return (tokens / bm + num_groups) * tiles_n;
 }
 
 }  // namespace
@@ -150,10 +177,12 @@ const char* gg_last_error(void) { return g_err; }
 
 int gg_version(void) { return 100; }
 
-int gg_tile_shape(int trans_a, int trans_b, int* bm, int* bn, int* bk) {
+int gg_tile_shape(int64_t num_groups, int64_t tokens, int trans_a, int trans_b, int* bm, int* bn,
+                  int* bk) {
   if (trans_a && trans_b) return fail(GG_EINVAL, "trans_a and trans_b cannot both be set");
-  if (bm) *bm = BM;
-  if (bn) *bn = BN;
+  const bool s = use_short_shape(num_groups, tokens, trans_a);
+  if (bm) *bm = s ? Short::BM : Wide::BM;
+  if (bn) *bn = s ? Short::BN : Wide::BN;
   if (bk) *bk = BK;
   return GG_OK;
 }
@@ -185,19 +214,17 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
   p.group_m = GG_GROUP_M;
   p.sched_out = nullptr;
 
+  const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
+  const int bm = short_shape ? Short::BM : Wide::BM, bn = short_shape ? Short::BN : Wide::BN;
   if (batch_sizes_on_device) {
-    if (tile_bound(num_groups, tokens, hidden_in, hidden_out, trans_a) >= (int64_t(1) << 31))
+    if (tile_bound(num_groups, tokens, hidden_in, hidden_out, trans_a, bm, bn) >= (int64_t(1) << 31))
       return fail(GG_ELIMIT, "too many output tiles for one launch");
     p.a = static_cast<const char*>(a);
     p.b = static_cast<const char*>(b);
     p.c = static_cast<char*>(c);
     p.sizes_dev = batch_sizes;
     p.num_groups = (int32_t)num_groups;
-    switch (layout) {
-      case gg::kNN: return launch<gg::kNN, false>(p, nullptr, info.cus, stream);
-      case gg::kNT: return launch<gg::kNT, false>(p, nullptr, info.cus, stream);
-      default: return launch<gg::kTN, false>(p, nullptr, info.cus, stream);
-    }
+    return dispatch<false>(short_shape, layout, p, nullptr, info.cus, stream);
   }
 
   // Host-resident sizes: validated here, passed in the kernel argument block, at most
@@ -215,12 +242,12 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
                               ? num_groups - first : GG_MAX_GROUPS_PER_LAUNCH;
     gg::HostSizes hs;
     int64_t rows_here = 0, tiles = 0;
-    const int64_t tiles_n = (hidden_out + BN - 1) / BN;
+    const int64_t tiles_n = (hidden_out + bn - 1) / bn;
     for (int64_t i = 0; i < count; ++i) {
       hs.v[i] = (int32_t)batch_sizes[first + i];
       rows_here += batch_sizes[first + i];
-      tiles += trans_a ? ((hidden_in + BM - 1) / BM) * tiles_n
-                       : ((batch_sizes[first + i] + BM - 1) / BM) * tiles_n;
+      tiles += trans_a ? ((hidden_in + bm - 1) / bm) * tiles_n
+                       : ((batch_sizes[first + i] + bm - 1) / bm) * tiles_n;
     }
     if (tiles >= (int64_t(1) << 31)) return fail(GG_ELIMIT, "too many output tiles for one launch");
     // this launch sees its own groups as groups 0..count-1 of operands that start at `row`
@@ -237,11 +264,7 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
     }
     if (tiles > 0) {
       const int grid = (int)(tiles < info.cus ? tiles : info.cus);
-      switch (layout) {
-        case gg::kNN: rc = launch<gg::kNN, true>(p, &hs, grid, stream); break;
-        case gg::kNT: rc = launch<gg::kNT, true>(p, &hs, grid, stream); break;
-        default: rc = launch<gg::kTN, true>(p, &hs, grid, stream); break;
-      }
+      rc = dispatch<true>(short_shape, layout, p, &hs, grid, stream);
       if (rc != GG_OK) return rc;
     }
     row += rows_here;
@@ -270,13 +293,10 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   p.num_groups = (int32_t)num_groups;
   p.sched_out = table_out;
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
+  const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
   if (batch_sizes_on_device) {
     p.sizes_dev = batch_sizes;
-    switch (layout) {
-      case gg::kNN: return launch_dump<gg::kNN, false>(p, nullptr, stream);
-      case gg::kNT: return launch_dump<gg::kNT, false>(p, nullptr, stream);
-      default: return launch_dump<gg::kTN, false>(p, nullptr, stream);
-    }
+    return dispatch_dump<false>(short_shape, layout, p, nullptr, stream);
   }
   gg::HostSizes hs;
   for (int64_t i = 0; i < num_groups; ++i) {
@@ -284,11 +304,7 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
       return fail(GG_EINVAL, "batch_sizes[%lld] out of range", (long long)i);
     hs.v[i] = (int32_t)batch_sizes[i];
   }
-  switch (layout) {
-    case gg::kNN: return launch_dump<gg::kNN, true>(p, &hs, stream);
-    case gg::kNT: return launch_dump<gg::kNT, true>(p, &hs, stream);
-    default: return launch_dump<gg::kTN, true>(p, &hs, stream);
-  }
+  return dispatch_dump<true>(short_shape, layout, p, &hs, stream);
 }
 
 }  // extern "C"

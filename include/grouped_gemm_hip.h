@@ -83,8 +83,11 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device,
                       int64_t hidden_out, int trans_a, int trans_b, int64_t* table_out,
                       void* stream);
 
-/* Tile shape (rows, columns, depth) the kernel for this layout uses; for reports. */
-int gg_tile_shape(int trans_a, int trans_b, int* bm, int* bn, int* bk);
+/* Output tile (rows, columns) and depth slice the kernel uses for a call with these arguments
+ * (calls whose groups average few rows get a shorter tile); for reports and for checking the
+ * tile counts of gg_debug_schedule. */
+int gg_tile_shape(int64_t num_groups, int64_t tokens, int trans_a, int trans_b, int* bm, int* bn,
+                  int* bk);
 
 /* Message of the last failure on the calling thread ("" if none). */
 const char* gg_last_error(void);

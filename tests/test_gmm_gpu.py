@@ -314,7 +314,8 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
     assert np.array_equal(got[:, 11], np.array(sizes))
     lib = ctypes.CDLL(os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so"))
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    lib.gg_tile_shape(int(trans_a), int(trans_b), ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk))
+    lib.gg_tile_shape(ctypes.c_int64(len(sizes)), ctypes.c_int64(tokens), int(trans_a), int(trans_b),
+                      ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk))
     m, n = got[:, 0], got[:, 1]
     assert np.array_equal(got[:, 10], -(-m // bm.value) * -(-n // bn.value))
 

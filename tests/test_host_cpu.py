@@ -141,7 +141,10 @@ def test_c_abi_argument_errors_need_no_device():
     assert call(16, 24, 0, 0, tokens=1 << 31) == -2
     assert call(16, 24, 0, 0, e=0) == 0                       # nothing to do
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
-    assert lib.gg_tile_shape(0, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
+    assert lib.gg_tile_shape(i64(8), i64(32768), 0, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
+    assert (bm.value, bn.value, bk.value) == (256, 256, 64)
+    assert lib.gg_tile_shape(i64(256), i64(25600), 0, 1, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
+    assert bm.value == 128          # few rows per group: the shorter tile
     assert bm.value > 0 and bn.value > 0 and bk.value > 0
     assert lib.gg_version() >= 100
 
