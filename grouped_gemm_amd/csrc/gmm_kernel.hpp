@@ -635,7 +635,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     constexpr int FIRST_LOAD = decltype(first_load_tag)::value, LOADS = decltype(loads_tag)::value;
     static_for<SLOTS>([&](auto m_tag) {
       constexpr int m = decltype(m_tag)::value;
-      constexpr int i = m / NB, j = m % NB;
+      // serpentine over the blocks: consecutive MFMAs share one operand, also across rows
+      constexpr int i = m / NB, j = (i % 2 == 0) ? m % NB : NB - 1 - m % NB;
       // operands swapped: the result block is held transposed, so a lane owns four
       // consecutive columns of one output row
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
