@@ -636,7 +636,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     static_for<SLOTS>([&](auto m_tag) {
       constexpr int m = decltype(m_tag)::value;
       // serpentine over the blocks: consecutive MFMAs share one operand, also across rows
-      constexpr int i = m / NB, j = (i % 2 == 0) ? m % NB : NB - 1 - m % NB;
+      constexpr int j = m / MB, i = (j % 2 == 0) ? m % MB : MB - 1 - m % MB;
       // operands swapped: the result block is held transposed, so a lane owns four
       // consecutive columns of one output row
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
