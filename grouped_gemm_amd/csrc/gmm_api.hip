@@ -41,8 +41,14 @@ int fail(int code, const char* fmt, ...) {
 #define GG_SHORT_BELOW 112   // average rows per group below which the short shape is used
 #endif
 constexpr int BK = 64, STAGES = 2;
+#ifndef GG_WIDE_WAVES_M
+#define GG_WIDE_WAVES_M 2
+#endif
+#ifndef GG_WIDE_WAVES_N
+#define GG_WIDE_WAVES_N 2
+#endif
 struct Wide {
-  static constexpr int BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2;
+  static constexpr int BM = 256, BN = 256, WAVES_M = GG_WIDE_WAVES_M, WAVES_N = GG_WIDE_WAVES_N;
 };
 struct Short {
   static constexpr int BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
