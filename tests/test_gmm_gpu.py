@@ -285,6 +285,48 @@ def test_config5_deepseek_share_full_size_autograd(ops, oracle):
         fp64_rows_check(w.a.detach(), w.b.detach(), sizes, True, out.detach())
 
 
+def _random_cases(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    cases = []
+    for _ in range(n):
+        e = r(1, 12)
+        kind = r(0, 3)
+        if kind == 0:      # many tiny groups
+            sizes = [r(0, 9) for _ in range(e)]
+        elif kind == 1:    # around the tile heights
+            sizes = [r(0, 3) * 128 + r(-2, 2) for _ in range(e)]
+        elif kind == 2:    # one big group among empties
+            sizes = [0] * e
+            sizes[r(0, e - 1)] = r(200, 900)
+        else:
+            sizes = [r(0, 400) for _ in range(e)]
+        sizes = [max(0, s) for s in sizes]
+        cases.append((sizes, 8 * r(1, 40), 8 * r(1, 70)))
+    return cases
+
+
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_random_shapes_against_cpu_oracle(ops, oracle, layout):
+    # depths that are not multiples of 64, widths that are not multiples of 256, sizes around
+    # the tile heights, host- and device-resident sizes alternating
+    trans_a, trans_b = layout
+    for idx, (sizes, hin, hout) in enumerate(_random_cases(24, seed=17 + int(trans_a) + 2 * int(trans_b))):
+        _announce("random", layout, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+        else:
+            b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+        dev_bs = bs.cuda() if idx % 2 else bs
+        out = ops.backend.gmm(a.cuda(), b.cuda(), dev_bs, trans_a=trans_a, trans_b=trans_b)
+        want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
+        check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
+
+
 # ----------------------------------------------------------------- schedule, bit-exact
 
 SCHED_CASES = [
