@@ -65,6 +65,9 @@ struct Sched {
 
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor size used here
 constexpr uint32_t kRsrcFlags = 0x00020000u;   // raw buffer, 32-bit data format
+// Cache policy of the output stores: non-temporal.  The output is written once and never read by
+// this kernel, so it should not push operand lines that other tiles still share out of L2.
+constexpr int kStoreStreaming = 2;
 
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
@@ -750,7 +753,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
               const int row = wm * Cfg::WTM + i * 32 + r * 8 + out_row;
               const int col = ti.n0 + wn * Cfg::WTN + jp * 64 + out_chunk * 8;
               const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
-              __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, 0);
+              __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, kStoreStreaming);
             }
             // keep the conversion of one strip from being hoisted over the stores of the
             // previous one: few accumulators are live in vector registers at a time
@@ -767,7 +770,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
             for (int q = 0; q < 4; ++q) {
               const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
               const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
-              __builtin_amdgcn_raw_buffer_store_b64(take4(i, j, q), rc, off, 0, 0);
+              __builtin_amdgcn_raw_buffer_store_b64(take4(i, j, q), rc, off, 0, kStoreStreaming);
             }
             __builtin_amdgcn_sched_barrier(0);
           }
