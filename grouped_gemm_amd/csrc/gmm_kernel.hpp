@@ -397,15 +397,18 @@ struct WidthMajor {
 // A fragment is the operand of one 32x32x16 MFMA: lane l holds 8 depth values
 // 8*(l/32) .. +7 of row (or column) l % 32.
 
-template <int BK>
+// STRIDE: distance between the blocks a wave owns, in 32-wide blocks (the waves along a
+// dimension take blocks alternately when STRIDE is their number, contiguously when it is 1).
+template <int BK, int STRIDE>
 struct DepthMajorFrag {
   static constexpr int CPR = BK / 8;
   static constexpr int RP = (BK * 2 >= 256) ? 1 : 256 / (BK * 2);
+  static_assert((32 / RP) % CPR == 0, "blocks must share the swizzle of block 0");
   uint32_t off[BK / 16];   // lane offset per 16-deep step, block 0
 
-  __device__ __forceinline__ void setup(int wave_row0) {
+  __device__ __forceinline__ void setup(int first_row) {
     const int lane = threadIdx.x & 63;
-    const int row = wave_row0 + (lane & 31);
+    const int row = first_row + (lane & 31);
     const int sw = (row / RP) % CPR;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
@@ -413,24 +416,24 @@ struct DepthMajorFrag {
     }
   }
   __device__ __forceinline__ bf16x8 read(const char* tile, int ks, int blk) const {
-    return *reinterpret_cast<const bf16x8*>(tile + off[ks] + blk * 32 * (BK * 2));
+    return *reinterpret_cast<const bf16x8*>(tile + off[ks] + blk * (STRIDE * 32) * (BK * 2));
   }
 };
 
-template <int W, int BK, int NBLK>
+template <int W, int BK, int NBLK, int STRIDE>
 struct WidthMajorFrag {
   static constexpr int PITCH = W * 2;
   static constexpr int SEGS = W * 2 / 64;
   uint32_t off[NBLK];   // lane offset per 32-wide block, depth step 0
 
-  __device__ __forceinline__ void setup(int wave_col0) {
+  __device__ __forceinline__ void setup(int first_col) {
     const int lane = threadIdx.x & 63;
     const int l16 = lane & 15;
     const int krow = 8 * (lane >> 5) + (l16 >> 2);
     const int g = (krow & 3) | (SEGS >= 8 ? ((krow >> 1) & 4) : 0);
 #pragma unroll
     for (int j = 0; j < NBLK; ++j) {
-      const int seg = (wave_col0 >> 5) + j;
+      const int seg = (first_col >> 5) + j * STRIDE;
       off[j] = (uint32_t)(krow * PITCH + ((seg ^ g) << 6) + 32 * ((lane >> 4) & 1) + 8 * (l16 & 3));
     }
   }
@@ -482,6 +485,7 @@ struct TileInfo {
   GroupGeom g;
   int m0, n0;       // first row and column of the tile inside its group's output
   int rows_valid;   // rows of the tile that exist (0: no tile)
+  int blocks;       // 32-row blocks the tile's rows take (MFMAs are issued for these only)
   int nk;           // depth slices, at least 1 so that an empty group still stores zeros
   bool valid;
 };
@@ -495,6 +499,7 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   if (t >= total_tiles) {
     ti.g = GroupGeom{0, 0, 0, 0, 0, 0};
     ti.m0 = ti.n0 = ti.rows_valid = 0;
+    ti.blocks = 1;
     ti.nk = 1;
     ti.valid = false;
     return ti;
@@ -507,9 +512,15 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   const int tiles_m = (ti.g.m + BM - 1) / BM;
   int tm, tn;
   tile_coords(u, tiles_m, tiles_n, p.group_m, &tm, &tn);
-  ti.m0 = uniform(tm) * BM;
+  // The rows of a group are split evenly over its tiles, in whole 32-row blocks: 300 rows
+  // make two tiles of 160 (5 blocks each), not one of 256 and one of 44.  Tiles of a group then
+  // take the same time, and blocks without rows cost nothing.
+  int height = BM;
+  if (LAYOUT != kTN && tiles_m > 0) height = ((ti.g.m + tiles_m - 1) / tiles_m + 31) / 32 * 32;
+  ti.m0 = uniform(tm) * height;
   ti.n0 = uniform(tn) * BN;
-  ti.rows_valid = min(BM, ti.g.m - ti.m0);
+  ti.rows_valid = min(height, ti.g.m - ti.m0);
+  ti.blocks = LAYOUT == kTN ? BM / 32 : max(1, (ti.rows_valid + 31) / 32);
   const int nk = (ti.g.k + BK - 1) / BK;
   ti.nk = nk < 1 ? 1 : nk;
   ti.valid = true;
@@ -524,14 +535,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB, KS = BK / 16;
   using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT>, WidthMajor<BM, BK, NT>>;
   using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT>, WidthMajor<BN, BK, NT>>;
-  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BM, BK, MB>>;
-  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK>, WidthMajorFrag<BN, BK, NB>>;
+  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK, WAVES_M>, WidthMajorFrag<BM, BK, MB, WAVES_M>>;
+  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK, 1>, WidthMajorFrag<BN, BK, NB, 1>>;
   constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;   // per lane, per depth slice
   constexpr int QUARTER_LOADS = LOADS_PER_STAGE / 4;
   static_assert(KS == 4 && STAGES == 2, "the step schedule below is written for BK = 64 and two buffers");
   static_assert(LOADS_PER_STAGE % 4 == 0 && LOADS_PER_STAGE < 32, "");
-  constexpr int UNITS = MB + NB;    // fragments read per 16-deep step
-  constexpr int SLOTS = MB * NB;    // MFMAs per 16-deep step
+  constexpr int UNITS = MB + NB;    // fragments of one 16-deep step
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   Sched* sched = reinterpret_cast<Sched*>(smem + Cfg::SCHED_OFFSET);
@@ -544,7 +554,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
 
   AFrag afrag;
   BFrag bfrag;
-  afrag.setup(wm * Cfg::WTM);
+  afrag.setup(wm * 32);   // wave row wm owns row blocks wm, wm + WAVES_M, ...
   bfrag.setup(wn * Cfg::WTN);
 
   const int total_tiles = uniform(sched->tile_start[p.num_groups]);
@@ -605,62 +615,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   };
 
   // Fragments: one register set per 16-deep step of a slice.  A "unit" is one fragment (one
-  // ds_read_b128, or two transposing 64-bit reads): A's MB first, then B's NB.
+  // ds_read_b128, or two transposing 64-bit reads): the first ML of A's, then B's NB.
   bf16x8 fa[KS][MB], fb[KS][NB];
-  auto read_unit = [&](auto u_tag, auto set_tag, int buf) {   // set = 16-deep step it belongs to
-    constexpr int U = decltype(u_tag)::value, SET = decltype(set_tag)::value;
+  auto read_unit = [&](auto u_tag, auto set_tag, auto ml_tag, int buf) {   // set = 16-deep step it belongs to
+    constexpr int U = decltype(u_tag)::value, SET = decltype(set_tag)::value, ML = decltype(ml_tag)::value;
     const char* sa = smem + buf * Cfg::STAGE_BYTES;
-    if constexpr (U < MB) {
+    if constexpr (U < ML) {
       fa[SET][U] = afrag.read(sa, SET, U);
     } else {
-      fb[SET][U - MB] = bfrag.read(sa + Cfg::A_BYTES, SET, U - MB);
+      fb[SET][U - ML] = bfrag.read(sa + Cfg::A_BYTES, SET, U - ML);
     }
   };
 
-  f32x16 acc[MB][NB];
-  auto zero_acc = [&]() {
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-      for (int j = 0; j < NB; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-  };
-
-  // One 16-deep step: SLOTS slots of one MFMA each, with this step's LDS reads and global
-  // loads placed behind the first MFMAs, in this order, so they run under the matrix pipe.
-  //   READS   fragments to fetch: unit u < UNITS goes to set READ_SET, units beyond to READ_SET+1
-  //   LOADS   global loads FIRST_LOAD .. of the fetch cursor's slice, into buffer `fill`
-  auto step = [&](auto ks_tag, auto reads_tag, auto read_set_tag, auto first_load_tag,
-                  auto loads_tag, int src, int fill) {
-    constexpr int ks = decltype(ks_tag)::value, READS = decltype(reads_tag)::value;
-    constexpr int READ_SET = decltype(read_set_tag)::value;
-    constexpr int FIRST_LOAD = decltype(first_load_tag)::value, LOADS = decltype(loads_tag)::value;
-    static_for<SLOTS>([&](auto m_tag) {
-      constexpr int m = decltype(m_tag)::value;
-      // serpentine over the blocks: consecutive MFMAs share one operand, also across rows
-      constexpr int j = m / MB, i = (j % 2 == 0) ? m % MB : MB - 1 - m % MB;
-      // operands swapped: the result block is held transposed, so a lane owns four
-      // consecutive columns of one output row
-      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
-      constexpr int u0 = READS * m / SLOTS, u1 = READS * (m + 1) / SLOTS;
-      static_for<u1 - u0>([&](auto d) {
-        constexpr int u = u0 + decltype(d)::value;
-        read_unit(std::integral_constant<int, u % UNITS>{},
-                  std::integral_constant<int, READ_SET + u / UNITS>{}, src);
-      });
-      constexpr int l0 = LOADS * m / SLOTS, l1 = LOADS * (m + 1) / SLOTS;
-      static_for<l1 - l0>([&](auto d) {
-        fetch_load(std::integral_constant<int, FIRST_LOAD + l0 + decltype(d)::value>{}, fill);
-      });
-      __builtin_amdgcn_sched_barrier(0);
-    });
-  };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
   using I2 = std::integral_constant<int, 2>;
   using I3 = std::integral_constant<int, 3>;
-  using IU2 = std::integral_constant<int, 2 * UNITS>;
+  using IMB = std::integral_constant<int, MB>;
   using IQ = std::integral_constant<int, QUARTER_LOADS>;
   using IQ2 = std::integral_constant<int, 2 * QUARTER_LOADS>;
   using IQ3 = std::integral_constant<int, 3 * QUARTER_LOADS>;
@@ -681,34 +652,80 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
     constexpr int uu = decltype(u)::value;
-    read_unit(std::integral_constant<int, uu % UNITS>{}, std::integral_constant<int, uu / UNITS>{}, 0);
+    read_unit(std::integral_constant<int, uu % UNITS>{}, std::integral_constant<int, uu / UNITS>{}, IMB{}, 0);
   });
 
+  int x = 0;   // buffer of the slice being multiplied
+
+  // One tile, for a wave that has ML row blocks with rows in them (the tile's row blocks go to
+  // the wave rows alternately).  One copy of this body exists per value of ML; a tile picks
+  // its copy once, so no accumulator ever lives across a choice.
+  //
   // Per slice (buffer X, the other buffer Y holds the next slice):
   //   step 0  reads the fragments of steps 2 and 3 from X; after it nobody needs X any more
   //   step 1  barrier: X goes to the fetch cursor, which starts the slice two ahead into it
   //   step 3  barrier: Y is complete for every wave; reads the fragments of the next slice's
-  //           steps 0 and 1 from Y
+  //           steps 0 and 1 from Y (all MB of A's: the next slice may be the next tile's)
   // Every step issues a quarter of a slice's loads (step 0 the last quarter of the slice begun
   // in steps 1-3 before it), so the memory pipe sees a steady trickle, and X is released two
   // steps before Y is needed, so loads stay in flight across the hand-over.
-  int x = 0;   // buffer of the slice being multiplied
-  while (true) {
-    zero_acc();
+  auto tile_body = [&](auto ml_tag) {
+    constexpr int ML = decltype(ml_tag)::value;
+    constexpr int SLOTS = ML * NB;    // MFMAs per 16-deep step
+    f32x16 acc[ML][NB];
+#pragma unroll
+    for (int i = 0; i < ML; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    // One 16-deep step: SLOTS slots of one MFMA each, with this step's LDS reads and global
+    // loads placed behind the first MFMAs, in this order, so they run under the matrix pipe.
+    //   RML     A fragments per set that are read (ML, or MB for the next slice's)
+    //   SETS    sets read: 0 or 2, starting at READ_SET
+    //   LOADS   global loads FIRST_LOAD .. of the fetch cursor's slice, into buffer `fill`
+    auto step = [&](auto ks_tag, auto sets_tag, auto rml_tag, auto read_set_tag, auto first_load_tag,
+                    auto loads_tag, int src, int fill) {
+      constexpr int ks = decltype(ks_tag)::value, SETS = decltype(sets_tag)::value;
+      constexpr int RML = decltype(rml_tag)::value, RUNITS = RML + NB, READS = SETS * RUNITS;
+      constexpr int READ_SET = decltype(read_set_tag)::value;
+      constexpr int FIRST_LOAD = decltype(first_load_tag)::value, LOADS = decltype(loads_tag)::value;
+      static_for<SLOTS>([&](auto m_tag) {
+        constexpr int m = decltype(m_tag)::value;
+        // serpentine over the blocks: consecutive MFMAs share one operand, also across rows
+        constexpr int j = m / ML, i = (j % 2 == 0) ? m % ML : ML - 1 - m % ML;
+        // operands swapped: the result block is held transposed, so a lane owns four
+        // consecutive columns of one output row
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+        constexpr int u0 = READS * m / SLOTS, u1 = READS * (m + 1) / SLOTS;
+        static_for<u1 - u0>([&](auto d) {
+          constexpr int u = u0 + decltype(d)::value;
+          read_unit(std::integral_constant<int, u % RUNITS>{},
+                    std::integral_constant<int, READ_SET + u / RUNITS>{}, rml_tag, src);
+        });
+        constexpr int l0 = LOADS * m / SLOTS, l1 = LOADS * (m + 1) / SLOTS;
+        static_for<l1 - l0>([&](auto d) {
+          fetch_load(std::integral_constant<int, FIRST_LOAD + l0 + decltype(d)::value>{}, fill);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    };
+
     for (int kt = 0; kt < ti.nk; ++kt) {
       const int y = x ^ 1;
-      step(I0{}, IU2{}, I2{}, IQ3{}, IQ{}, x, y);
+      step(I0{}, I2{}, ml_tag, I2{}, IQ3{}, IQ{}, x, y);
       fetch_advance();
       // every wave has all fragments of this slice in registers
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
       block_barrier();
       fetch_begin();
-      step(I1{}, I0{}, I0{}, I0{}, IQ{}, x, x);
-      step(I2{}, I0{}, I0{}, IQ{}, IQ{}, x, x);
+      step(I1{}, I0{}, ml_tag, I0{}, I0{}, IQ{}, x, x);
+      step(I2{}, I0{}, ml_tag, I0{}, IQ{}, IQ{}, x, x);
       // the next slice has landed for every wave (only this slice's two quarters may be pending)
       wait_vmcnt<2 * QUARTER_LOADS>();
       block_barrier();
-      step(I3{}, IU2{}, I0{}, IQ2{}, IQ{}, y, x);
+      step(I3{}, I2{}, IMB{}, I0{}, IQ2{}, IQ{}, y, x);
       x = y;
     }
 
@@ -738,7 +755,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
         const int in_row = lane & 31, in_half = lane >> 5;
         const int out_row = lane >> 3, out_chunk = lane & 7;
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
+        for (int i = 0; i < ML; ++i) {
 #pragma unroll
           for (int jp = 0; jp < NB / 2; ++jp) {
 #pragma unroll
@@ -750,7 +767,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const u32x4 v = *reinterpret_cast<const u32x4*>(strip + (r * 8 + out_row) * PITCH + out_chunk * 16);
-              const int row = wm * Cfg::WTM + i * 32 + r * 8 + out_row;
+              const int row = (wm + i * WAVES_M) * 32 + r * 8 + out_row;
               const int col = ti.n0 + wn * Cfg::WTN + jp * 64 + out_chunk * 8;
               const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
               __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, kStoreStreaming);
@@ -762,8 +779,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
         }
       } else {
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-          const int row = wm * Cfg::WTM + i * 32 + (lane & 31);
+        for (int i = 0; i < ML; ++i) {
+          const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
 #pragma unroll
           for (int j = 0; j < NB; ++j) {
 #pragma unroll
@@ -775,6 +792,25 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
             __builtin_amdgcn_sched_barrier(0);
           }
         }
+      }
+    }
+  };
+
+  while (true) {
+    // row blocks of this tile that fall to this wave row: blocks wm, wm + WAVES_M, ...
+    const int live = uniform((ti.blocks - wm + WAVES_M - 1) / WAVES_M);
+    if constexpr (LAYOUT == kTN || MB == 1) {
+      tile_body(IMB{});
+    } else {
+      static_assert(MB == 4, "one copy of the tile body per live block count 1..4");
+      if (live >= 4) {
+        tile_body(std::integral_constant<int, 4>{});
+      } else if (live == 3) {
+        tile_body(std::integral_constant<int, 3>{});
+      } else if (live == 2) {
+        tile_body(std::integral_constant<int, 2>{});
+      } else {
+        tile_body(std::integral_constant<int, 1>{});
       }
     }
     tile_t += G;
