@@ -327,6 +327,37 @@ def test_random_shapes_against_cpu_oracle(ops, oracle, layout):
         check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("on_device", [False, True])
+def test_every_row_block_count(ops, oracle, trans_b, on_device):
+    # One call whose groups cover every count of 32-row blocks a tile can have, on both sides of
+    # each boundary, and groups whose rows are split evenly over two, three and five tiles; the
+    # value of each output row names its input row, so a row that lands in the wrong place shows.
+    sizes = [1, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 159, 160, 161, 191, 192, 193,
+             223, 224, 225, 255, 256, 257, 289, 300, 320, 321, 511, 512, 513, 700, 0, 1025, 1281]
+    hin, hout = 192, 328
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    t = int(bs.sum())
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+    _announce("row blocks", trans_b, on_device)
+    out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda() if on_device else bs, trans_b=trans_b)
+    check(out, oracle.gmm_loop(a, b, bs, trans_b=trans_b), "every row block count")
+    # exact: one-hot rows times an identity-like weight give back the row index pattern
+    eye = torch.zeros(len(sizes), hin, hout)
+    eye[:, :, :hin] = torch.eye(hin)
+    wb = (eye.transpose(1, 2).contiguous() if trans_b else eye).to(torch.bfloat16)
+    idx = torch.arange(t) % 251
+    rows = torch.zeros(t, hin)
+    rows[torch.arange(t), idx % hin] = (idx % 127 + 1).float()
+    got = ops.backend.gmm(rows.to(torch.bfloat16).cuda(), wb.cuda(), bs.cuda() if on_device else bs,
+                          trans_b=trans_b).float().cpu()
+    want = torch.zeros(t, hout)
+    want[:, :hin] = rows
+    assert torch.equal(got, want)
+
+
 # ----------------------------------------------------------------- schedule, bit-exact
 
 SCHED_CASES = [
