@@ -6,6 +6,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -62,6 +63,12 @@ struct Wide {
 struct Short {
   static constexpr int BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
 };
+
+// GG_TAIL_SPLIT=0 in the environment keeps the tiles of the last round whole (read at every call).
+int tail_split() {
+  const char* e = getenv("GG_TAIL_SPLIT");
+  return e != nullptr && e[0] == '0' ? 0 : 1;
+}
 
 int band_height(int64_t num_groups, int64_t tokens, int trans_a) {
   return trans_a && tokens < (int64_t)GG_SHALLOW_BELOW * num_groups ? GG_GROUP_M_SHALLOW : GG_GROUP_M;
@@ -231,6 +238,7 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
   p.hidden_in = (int32_t)hidden_in;
   p.hidden_out = (int32_t)hidden_out;
   p.group_m = band_height(num_groups, tokens, trans_a);
+  p.tail_split = tail_split();
   p.sched_out = nullptr;
 
   const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
@@ -282,8 +290,9 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
       p.c = static_cast<char*>(c) + row * hidden_out * 2;
     }
     if (tiles > 0) {
-      const int grid = (int)(tiles < info.cus ? tiles : info.cus);
-      rc = dispatch<true>(short_shape, layout, p, &hs, grid, stream);
+      // the full grid also for few tiles: the last round's tiles may be cut into pieces for
+      // the workgroups that would otherwise idle
+      rc = dispatch<true>(short_shape, layout, p, &hs, info.cus, stream);
       if (rc != GG_OK) return rc;
     }
     row += rows_here;
@@ -309,6 +318,7 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   p.hidden_in = (int32_t)hidden_in;
   p.hidden_out = (int32_t)hidden_out;
   p.group_m = band_height(num_groups, tokens, trans_a);
+  p.tail_split = tail_split();
   p.num_groups = (int32_t)num_groups;
   p.sched_out = table_out;
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);

@@ -48,7 +48,27 @@ struct GmmParams {
   int32_t hidden_in;
   int32_t hidden_out;
   int32_t group_m;  // tile rows per band of the in-group tile order
+  int32_t tail_split;  // 1: the tiles of the last, partly filled round may be cut into row pieces
 };
+
+// The last round of a persistent grid is filled only partly: `tiles % grid` workgroups have a
+// tile, the others idle.  When that rest is at most half (a quarter) of the grid, each of its
+// tiles is cut along its rows into 2 (4) pieces that go to different workgroups; a piece issues
+// MFMAs only for its own 32-row blocks, so the round ends sooner.  A launch with fewer tiles
+// than workgroups is all "last round".
+struct TailPlan {
+  int main_tiles;   // tiles before the last round, handed out whole
+  int pieces;       // pieces per tile of the last round: 1, 2 or 4
+  int total;        // indices to hand out: main_tiles + rest * pieces
+};
+__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, bool enabled) {
+  TailPlan t;
+  const int rest = tiles % grid;
+  t.pieces = !enabled || rest == 0 ? 1 : (4 * rest <= grid ? 4 : (2 * rest <= grid ? 2 : 1));
+  t.main_tiles = t.pieces > 1 ? tiles - rest : tiles;
+  t.total = t.main_tiles + (tiles - t.main_tiles) * t.pieces;
+  return t;
+}
 
 // Host-resident batch_sizes travel in the kernel argument block: no copy, no staging.
 struct HostSizes {
@@ -486,23 +506,31 @@ struct TileInfo {
   int m0, n0;       // first row and column of the tile inside its group's output
   int rows_valid;   // rows of the tile that exist (0: no tile)
   int blocks;       // 32-row blocks the tile's rows take (MFMAs are issued for these only)
+  int depth;        // depth to fetch (0: nothing to fetch, the tile multiplies zeros)
   int nk;           // depth slices, at least 1 so that an empty group still stores zeros
   bool valid;
 };
 
 // Tile index -> group and position.  `e` is the caller's cursor into the groups; tile
-// indices only grow, so it only moves forward.
+// indices only grow, so it only moves forward.  Indices past plan.main_tiles name pieces of the
+// last round's tiles: piece (t - main) % pieces of tile main + (t - main) / pieces.
 template <int LAYOUT, int BM, int BN, int BK>
 __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParams& p, int t,
-                                              int total_tiles, int& e) {
+                                              const TailPlan& plan, int& e) {
   TileInfo ti;
-  if (t >= total_tiles) {
+  if (t >= plan.total) {
     ti.g = GroupGeom{0, 0, 0, 0, 0, 0};
-    ti.m0 = ti.n0 = ti.rows_valid = 0;
+    ti.m0 = ti.n0 = ti.rows_valid = ti.depth = 0;
     ti.blocks = 1;
     ti.nk = 1;
     ti.valid = false;
     return ti;
+  }
+  int piece = -1;
+  if (t >= plan.main_tiles) {
+    const int r = t - plan.main_tiles;
+    piece = r % plan.pieces;
+    t = plan.main_tiles + r / plan.pieces;
   }
   while (t >= uniform(sched->tile_start[e + 1])) ++e;
   // read through the first lane: everything derived from these stays in scalar registers
@@ -520,9 +548,23 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   ti.m0 = uniform(tm) * height;
   ti.n0 = uniform(tn) * BN;
   ti.rows_valid = min(height, ti.g.m - ti.m0);
-  ti.blocks = LAYOUT == kTN ? BM / 32 : max(1, (ti.rows_valid + 31) / 32);
+  ti.depth = ti.g.k;
   const int nk = (ti.g.k + BK - 1) / BK;
   ti.nk = nk < 1 ? 1 : nk;
+  if (piece >= 0) {
+    // this piece's share of the tile's 32-row blocks; a piece past the rows is an empty tile
+    const int all = (ti.rows_valid + 31) / 32;
+    const int per = (all + plan.pieces - 1) / plan.pieces;
+    const int skip = piece * per * 32;
+    ti.m0 += skip;
+    ti.rows_valid = min(per * 32, ti.rows_valid - skip);
+    if (ti.rows_valid <= 0) {
+      ti.rows_valid = 0;
+      ti.depth = 0;
+      ti.nk = 1;
+    }
+  }
+  ti.blocks = LAYOUT == kTN ? BM / 32 : max(1, (ti.rows_valid + 31) / 32);
   ti.valid = true;
   return ti;
 }
@@ -557,7 +599,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   afrag.setup(wm * 32);   // wave row wm owns row blocks wm, wm + WAVES_M, ...
   bfrag.setup(wn * Cfg::WTN);
 
-  const int total_tiles = uniform(sched->tile_start[p.num_groups]);
+  // (the weight-gradient layout has no ragged rows and no tile body for part of a tile)
+  const TailPlan plan = plan_tail(uniform(sched->tile_start[p.num_groups]), (int)gridDim.x,
+                                  LAYOUT != kTN && p.tail_split != 0);
+  const int total_tiles = plan.total;
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
   // tile indices so that its private L2 sees neighbouring tiles.
@@ -574,8 +619,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   int fetch_t = vid, fetch_e = 0, fetch_kt = 0;
   TileInfo fti;
   auto fetch_setup = [&]() {
-    fti = find_tile<LAYOUT, BM, BN, BK>(sched, p, fetch_t, total_tiles, fetch_e);
-    const int depth = fti.valid ? fti.g.k : 0;
+    fti = find_tile<LAYOUT, BM, BN, BK>(sched, p, fetch_t, plan, fetch_e);
+    const int depth = fti.depth;
     if constexpr (Cfg::A_DEPTH_MAJOR) {
       aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * 2, fti.g.k, fti.rows_valid, depth);
     } else {
@@ -583,7 +628,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     }
     if constexpr (Cfg::B_DEPTH_MAJOR) {
       bload.setup(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
-                  fti.valid ? min(BN, fti.g.n - fti.n0) : 0, depth);
+                  fti.valid && depth > 0 ? min(BN, fti.g.n - fti.n0) : 0, depth);
     } else {
       bload.setup(p.b + fti.g.b_off * 2, fti.g.n, depth, fti.n0, fti.g.n);
     }
@@ -647,7 +692,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   static_for<3 * QUARTER_LOADS>([&](auto j) { fetch_load(j, 1); });
 
   int tile_t = vid, tile_e = 0;
-  TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, total_tiles, tile_e);
+  TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_e);
   wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
@@ -815,7 +860,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     }
     tile_t += G;
     if (tile_t >= total_tiles) break;
-    ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, total_tiles, tile_e);
+    ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_e);
   }
   wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
 #endif  // __HIP_DEVICE_COMPILE__

@@ -358,6 +358,28 @@ def test_every_row_block_count(ops, oracle, trans_b, on_device):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_last_round_pieces_equal_whole_tiles(ops, oracle, trans_b, monkeypatch):
+    # A launch with fewer tiles than workgroups cuts its tiles into row pieces for the idle
+    # workgroups; GG_TAIL_SPLIT=0 keeps them whole.  Same depth order per output element either
+    # way, so the two must agree bit for bit (and with the oracle within tolerance).
+    for idx, (sizes, hin, hout) in enumerate(_random_cases(16, seed=91 + int(trans_b))):
+        _announce("pieces", trans_b, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
+        b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16).cuda()
+        dev_bs = bs.cuda() if idx % 2 else bs
+        monkeypatch.setenv("GG_TAIL_SPLIT", "1")
+        cut = ops.backend.gmm(a, b, dev_bs, trans_b=trans_b)
+        monkeypatch.setenv("GG_TAIL_SPLIT", "0")
+        whole = ops.backend.gmm(a, b, dev_bs, trans_b=trans_b)
+        assert torch.equal(cut, whole), f"case {idx}: sizes={sizes} hin={hin} hout={hout}"
+        check(whole, oracle.gmm_loop(a.cpu(), b.cpu(), bs, trans_b=trans_b), f"case {idx}")
+    monkeypatch.delenv("GG_TAIL_SPLIT")
+
+
 # ----------------------------------------------------------------- schedule, bit-exact
 
 SCHED_CASES = [
