@@ -31,8 +31,8 @@ PEAK_HBM_GBPS = 8000.0
 # runs of this file (FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by a 1 GiB device copy, both in
 # KiB); the figures and commands are in profiles/gmm_kernel_mixtral_w1_hbm_traffic.md.
 MEASURED_TRAFFIC_BYTES = {
-    2: {"fwd": (3097005 * 2.0 + 917504) * 1024, "agrad": (3256868 * 2.0 + 262144) * 1024,
-        "bgrad": (2753228 * 2.0 + 917504) * 1024},
+    2: {"fwd": (4458000 * 2.0 + 917600) * 1024, "agrad": (3812000 * 2.0 + 262144) * 1024,
+        "bgrad": (2755000 * 2.0 + 917500) * 1024},
 }
 
 
@@ -86,8 +86,8 @@ def cpu_baseline(w, budget_s=12.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration (2 = Mixtral w1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--zeros", action="store_true",
@@ -154,7 +154,8 @@ def main():
     bytes_gemm = w.bytes_per_gemm()
     ms_per_step = elapsed / args.steps * 1e3
     value = flops_gemm * len(names) / (ms_per_step * 1e-3) / 1e12
-    kernel_ms = {n: sum(a.elapsed_time(b) for a, b in ev) / len(ev) for n, ev in events.items()}
+    samples = {n: sorted(a.elapsed_time(b) for a, b in ev) for n, ev in events.items()}
+    kernel_ms = {n: sum(v) / len(v) for n, v in samples.items()}
     slowest = max(kernel_ms, key=kernel_ms.get)
     achieved = flops_gemm / (kernel_ms[slowest] * 1e-3) / 1e12
 
@@ -193,6 +194,8 @@ def main():
             "per_kernel": {
                 f"{layout[n]} ({n})": {
                     "ms": round(ms, 4),
+                    "median_ms": round(samples[n][len(samples[n]) // 2], 4),
+                    "min_ms": round(samples[n][0], 4),
                     "TFLOP/s": round(flops_gemm / (ms * 1e-3) / 1e12, 2),
                     "frac_mfma": round(flops_gemm / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
                     "GB/s": round(bytes_gemm / (ms * 1e-3) / 1e9, 1),
