@@ -223,6 +223,9 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
   if (hidden_out == 0 || (trans_a ? hidden_in == 0 : tokens == 0)) return GG_OK;
   if (c == nullptr) return fail(GG_EINVAL, "c is null");
   if (tokens > 0 && (a == nullptr || b == nullptr)) return fail(GG_EINVAL, "a or b is null");
+  // rows are fetched and stored 16 bytes at a time
+  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15)
+    return fail(GG_ELIMIT, "a, b and c must be 16-byte aligned");
   if (batch_sizes_on_device && num_groups > GG_MAX_GROUPS_PER_LAUNCH)
     return fail(GG_ELIMIT, "at most %d groups are supported when batch_sizes is on the device, got %lld",
                 GG_MAX_GROUPS_PER_LAUNCH, (long long)num_groups);

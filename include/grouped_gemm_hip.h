@@ -58,9 +58,9 @@ extern "C" {
  * vector can make the kernel read or write outside a, b or c.
  * stream: a hipStream_t (NULL = the default stream).
  *
- * Limits (GG_ELIMIT): hidden_in and hidden_out multiples of 8 (16-byte rows, the same
- * alignment the reference's kernel configuration assumes, csrc/grouped_gemm.cu:41-66)
- * and below 2^22; tokens below 2^31; num_groups <= GG_MAX_GROUPS_PER_LAUNCH when
+ * Limits (GG_ELIMIT): a, b and c 16-byte aligned, hidden_in and hidden_out multiples of 8
+ * (16-byte rows, the same alignment the reference's kernel configuration assumes,
+ * csrc/grouped_gemm.cu:41-66) and below 2^22; tokens below 2^31; num_groups <= GG_MAX_GROUPS_PER_LAUNCH when
  * batch_sizes is on the device.
  */
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,

@@ -140,6 +140,11 @@ def test_c_abi_argument_errors_need_no_device():
     assert call(-8, 24, 0, 0) == -1
     assert call(16, 24, 0, 0, tokens=1 << 31) == -2
     assert call(16, 24, 0, 0, e=0) == 0                       # nothing to do
+    # fake, never dereferenced pointers: the alignment check comes before any device call
+    ptr = ctypes.c_void_p
+    misaligned = lib.gg_gmm_bf16(ptr(4096), ptr(8192 + 2), ptr(12288), sizes, 0, i64(2), i64(8), i64(16),
+                                 i64(24), 0, 0, None)
+    assert misaligned == -2 and b"16-byte aligned" in lib.gg_last_error()
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     assert lib.gg_tile_shape(i64(8), i64(32768), 0, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
     assert (bm.value, bn.value, bk.value) == (256, 256, 64)
