@@ -478,6 +478,53 @@ def test_c_abi_rejects_bad_host_sizes():
     assert rc == -2 and b"512" in lib.gg_last_error()
 
 
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_groups_are_isolated_from_each_other(ops, layout):
+    # NaNs in the rows of one group (and in its weights) must show up in that group's output
+    # only: tiles are cut at group ends by the buffer descriptors, never by arithmetic on
+    # neighbouring rows.  Sizes straddle every tile and block boundary.
+    trans_a, trans_b = layout
+    sizes = [70, 1, 0, 300, 129, 255]
+    poisoned = 3
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    starts = [0] + list(torch.cumsum(bs, 0))
+    t, hin, hout = int(bs.sum()), 136, 264
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    a[starts[poisoned]:starts[poisoned + 1]] = float("nan")
+    if trans_a:
+        b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+    else:
+        b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+        b[poisoned] = float("nan")
+    _announce("isolation", layout)
+    out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda(), trans_a=trans_a, trans_b=trans_b).float().cpu()
+    for e in range(len(sizes)):
+        block = out[e] if trans_a else out[starts[e]:starts[e + 1]]
+        if e == poisoned:
+            assert torch.isnan(block).all()
+        else:
+            assert not torch.isnan(block).any(), e
+
+
+def test_repeated_calls_are_bitwise_identical(ops):
+    # no atomics, no split accumulation: the same call gives the same bits every time
+    w_sizes = torch.tensor([300, 0, 17, 1000, 256, 129], dtype=torch.int64)
+    t = int(w_sizes.sum())
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn(t, 520, generator=g).to(torch.bfloat16).cuda()
+    b = torch.randn(6, 520, 776, generator=g).to(torch.bfloat16).cuda()
+    grad = torch.randn(t, 776, generator=g).to(torch.bfloat16).cuda()
+    sd = w_sizes.cuda()
+    first = [ops.backend.gmm(a, b, sd), ops.backend.gmm(grad, b, sd, trans_b=True),
+             ops.backend.gmm(a, grad, sd, trans_a=True)]
+    for _ in range(5):
+        again = [ops.backend.gmm(a, b, sd), ops.backend.gmm(grad, b, sd, trans_b=True),
+                 ops.backend.gmm(a, grad, sd, trans_a=True)]
+        for x, y in zip(first, again):
+            assert torch.equal(x, y)
+
+
 # ------------------------------------------------------------------------ edge cases
 
 def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):
