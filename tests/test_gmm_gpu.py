@@ -525,6 +525,44 @@ def test_repeated_calls_are_bitwise_identical(ops):
             assert torch.equal(x, y)
 
 
+def test_hip_graph_replay_with_new_device_sizes(ops, oracle):
+    # The call allocates nothing and never reads batch_sizes on the host when they live on the
+    # device, so it can be captured in a HIP graph once and replayed with other group sizes:
+    # the kernel re-derives its schedule from the size buffer at every replay.  Replays are
+    # interleaved with eager work and checked one by one.
+    hin, hout, t = 256, 392, 1500
+    g = torch.Generator().manual_seed(23)
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
+    b = torch.randn(5, hin, hout, generator=g).to(torch.bfloat16).cuda()
+    grad = torch.randn(t, hout, generator=g).to(torch.bfloat16).cuda()
+    sizes = torch.tensor([300, 300, 300, 300, 300], dtype=torch.int64).cuda()
+    out = torch.empty(t, hout, dtype=torch.bfloat16, device="cuda")
+    wgrad = torch.empty(5, hin, hout, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):      # warm-up outside the capture (first-call attribute setting)
+        ops.backend.gmm(a, b, sizes, c=out)
+        ops.backend.gmm(a, grad, sizes, trans_a=True, c=wgrad)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.backend.gmm(a, b, sizes, c=out)
+        ops.backend.gmm(a, grad, sizes, trans_a=True, c=wgrad)
+    for new_sizes in ([300] * 5, [1500, 0, 0, 0, 0], [1, 2, 3, 4, 1490], [0, 700, 0, 800, 0], [299, 301, 17, 600, 283]):
+        _announce("graph replay", new_sizes)
+        sizes.copy_(torch.tensor(new_sizes, dtype=torch.int64))
+        out.fill_(7.0)
+        wgrad.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = ops.backend.gmm(a, b, sizes)
+        eager_w = ops.backend.gmm(a, grad, sizes, trans_a=True)
+        assert torch.equal(out, eager), new_sizes
+        assert torch.equal(wgrad, eager_w), new_sizes
+        check(out, oracle.gmm_loop(a.cpu(), b.cpu(), torch.tensor(new_sizes)), f"replay {new_sizes}")
+
+
 # ------------------------------------------------------------------------ edge cases
 
 def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):
