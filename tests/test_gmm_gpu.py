@@ -563,6 +563,31 @@ def test_hip_graph_replay_with_new_device_sizes(ops, oracle):
         check(out, oracle.gmm_loop(a.cpu(), b.cpu(), torch.tensor(new_sizes)), f"replay {new_sizes}")
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_traceable_operator_under_torch_compile(ops, trans_b):
+    # one graph, no breaks (fullgraph), forward and both gradients bit-equal to the autograd
+    # Function of the reference's surface
+    sizes = torch.tensor([37, 0, 300, 163], dtype=torch.int64).cuda()
+    g = torch.Generator().manual_seed(29)
+    a0 = torch.randn(500, 136, generator=g).to(torch.bfloat16).cuda()
+    b0 = torch.randn(4, *((200, 136) if trans_b else (136, 200)), generator=g).to(torch.bfloat16).cuda()
+    grad = torch.randn(500, 200, generator=g).to(torch.bfloat16).cuda()
+
+    def run(fn):
+        a, b = a0.clone().requires_grad_(), b0.clone().requires_grad_()
+        out = fn(a, b)
+        out.backward(grad)
+        return out.detach(), a.grad, b.grad
+
+    eager = run(lambda a, b: ops.gmm(a, b, sizes, trans_b))
+    compiled_fn = torch.compile(lambda a, b: ops.gmm_traceable(a, b, sizes, trans_b) * 1.0,
+                                backend="aot_eager", fullgraph=True)
+    _announce("torch.compile", trans_b)
+    compiled = run(compiled_fn)
+    for x, y in zip(eager, compiled):
+        assert torch.equal(x, y)
+
+
 # ------------------------------------------------------------------------ edge cases
 
 def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):

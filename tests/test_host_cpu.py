@@ -191,3 +191,20 @@ def test_config1_fixture_matches_oracle(oracle):
     torch.testing.assert_close(out, fwd, rtol=1e-5, atol=1e-4)
     torch.testing.assert_close(ag, agrad, rtol=1e-5, atol=1e-4)
     torch.testing.assert_close(bg, bgrad, rtol=1e-5, atol=1e-4)
+
+
+# ----------------------------------------------------------------- traceable operator
+
+def test_traceable_operator_shapes_without_a_device():
+    # the torch.library form of the operator: output shapes for all three layouts from fake
+    # tensors alone (what torch.compile needs), no kernel runs
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from grouped_gemm_amd import ops
+    with FakeTensorMode():
+        a = torch.empty(100, 64, dtype=torch.bfloat16)
+        bs = torch.empty(4, dtype=torch.int64)
+        assert ops.gmm_traceable(a, torch.empty(4, 64, 96, dtype=torch.bfloat16), bs).shape == (100, 96)
+        assert ops.gmm_traceable(a, torch.empty(4, 96, 64, dtype=torch.bfloat16), bs, trans_b=True).shape == (100, 96)
+        wgrad = torch.ops.grouped_gemm_amd.gmm(a, torch.empty(100, 96, dtype=torch.bfloat16), bs, True, False)
+        assert wgrad.shape == (4, 64, 96) and wgrad.dtype == torch.bfloat16
+
