@@ -102,12 +102,12 @@ int device_info(DeviceInfo* out) {
   return GG_OK;
 }
 
-template <typename S, int LAYOUT, bool HOST_SIZES>
+template <typename S, int LAYOUT, bool HOST_SIZES, bool ACC_F32 = false>
 int launch(const gg::GmmParams& p, const gg::HostSizes* hs, int grid, hipStream_t stream) {
   using Cfg = gg::GmmConfig<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N>;
   constexpr int kThreads = S::WAVES_M * S::WAVES_N * 64;
   const void* kernel = reinterpret_cast<const void*>(
-      &gg::gmm_kernel<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, HOST_SIZES>);
+      &gg::gmm_kernel<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, HOST_SIZES, ACC_F32>);
   // raising the dynamic LDS limit is per device and per kernel; do it once each
   static std::mutex mu;
   static bool done[64] = {};
@@ -148,9 +148,11 @@ int launch_dump(const gg::GmmParams& p, const gg::HostSizes* hs, hipStream_t str
   return GG_OK;
 }
 
+// out_f32: the accumulating form (weight-gradient layout only).
 template <bool HOST_SIZES>
-int dispatch(bool short_shape, int layout, const gg::GmmParams& p, const gg::HostSizes* hs, int grid,
-             hipStream_t stream) {
+int dispatch(bool short_shape, int layout, bool out_f32, const gg::GmmParams& p, const gg::HostSizes* hs,
+             int grid, hipStream_t stream) {
+  if (out_f32) return launch<Wide, gg::kTN, HOST_SIZES, true>(p, hs, grid, stream);
   if (layout == gg::kTN) return launch<Wide, gg::kTN, HOST_SIZES>(p, hs, grid, stream);
   if (short_shape) {
     return layout == gg::kNN ? launch<Short, gg::kNN, HOST_SIZES>(p, hs, grid, stream)
@@ -195,6 +197,10 @@ int64_t tile_bound(int64_t num_groups, int64_t tokens, int64_t hidden_in, int64_
   return (tokens / bm + num_groups) * tiles_n;
 }
 
+int gmm_impl(const void* a, const void* b, void* c, bool out_f32, const int64_t* batch_sizes,
+             int batch_sizes_on_device, int64_t num_groups, int64_t tokens, int64_t hidden_in,
+             int64_t hidden_out, int trans_a, int trans_b, void* stream_);
+
 }  // namespace
 
 extern "C" {
@@ -216,6 +222,26 @@ int gg_tile_shape(int64_t num_groups, int64_t tokens, int trans_a, int trans_b, 
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,
                 int batch_sizes_on_device, int64_t num_groups, int64_t tokens, int64_t hidden_in,
                 int64_t hidden_out, int trans_a, int trans_b, void* stream_) {
+  return gmm_impl(a, b, c, /*out_f32=*/false, batch_sizes, batch_sizes_on_device, num_groups, tokens,
+                  hidden_in, hidden_out, trans_a, trans_b, stream_);
+}
+
+int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* batch_sizes,
+                        int batch_sizes_on_device, int64_t num_groups, int64_t tokens,
+                        int64_t hidden_in, int64_t hidden_out, void* stream_) {
+  if (hidden_in >= (1 << 20) || hidden_out >= (1 << 20))
+    return fail(GG_ELIMIT, "hidden sizes must be below 2^20 for the accumulating form");
+  return gmm_impl(a, b, c, /*out_f32=*/true, batch_sizes, batch_sizes_on_device, num_groups, tokens,
+                  hidden_in, hidden_out, /*trans_a=*/1, /*trans_b=*/0, stream_);
+}
+
+}  // extern "C"
+
+namespace {
+
+int gmm_impl(const void* a, const void* b, void* c, bool out_f32, const int64_t* batch_sizes,
+             int batch_sizes_on_device, int64_t num_groups, int64_t tokens, int64_t hidden_in,
+             int64_t hidden_out, int trans_a, int trans_b, void* stream_) {
   int rc = check_common(batch_sizes, num_groups, tokens, hidden_in, hidden_out, trans_a, trans_b);
   if (rc != GG_OK) return rc;
   if (num_groups == 0) return GG_OK;
@@ -254,7 +280,7 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
     p.c = static_cast<char*>(c);
     p.sizes_dev = batch_sizes;
     p.num_groups = (int32_t)num_groups;
-    return dispatch<false>(short_shape, layout, p, nullptr, info.cus, stream);
+    return dispatch<false>(short_shape, layout, out_f32, p, nullptr, info.cus, stream);
   }
 
   // Host-resident sizes: validated here, passed in the kernel argument block, at most
@@ -287,7 +313,7 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
     p.a = static_cast<const char*>(a) + row * hidden_in * 2;
     if (trans_a) {
       p.b = static_cast<const char*>(b) + row * hidden_out * 2;
-      p.c = static_cast<char*>(c) + first * hidden_in * hidden_out * 2;
+      p.c = static_cast<char*>(c) + first * hidden_in * hidden_out * (out_f32 ? 4 : 2);
     } else {
       p.b = static_cast<const char*>(b) + first * hidden_in * hidden_out * 2;
       p.c = static_cast<char*>(c) + row * hidden_out * 2;
@@ -295,13 +321,17 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
     if (tiles > 0) {
       // the full grid also for few tiles: the last round's tiles may be cut into pieces for
       // the workgroups that would otherwise idle
-      rc = dispatch<true>(short_shape, layout, p, &hs, info.cus, stream);
+      rc = dispatch<true>(short_shape, layout, out_f32, p, &hs, info.cus, stream);
       if (rc != GG_OK) return rc;
     }
     row += rows_here;
   }
   return GG_OK;
 }
+
+}  // namespace
+
+extern "C" {
 
 int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int64_t num_groups,
                       int64_t tokens, int64_t hidden_in, int64_t hidden_out, int trans_a,

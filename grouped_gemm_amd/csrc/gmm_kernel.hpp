@@ -569,7 +569,10 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   return ti;
 }
 
-template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool HOST_SIZES>
+// ACC_F32: c holds fp32 and the product is added to it (gradient accumulation); otherwise c
+// holds bf16 and is overwritten.
+template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool HOST_SIZES,
+          bool ACC_F32 = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     GmmParams p, std::conditional_t<HOST_SIZES, HostSizes, NoSizes> hs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
@@ -778,8 +781,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     // The accumulators stay in the accumulation registers; each value is moved out right
     // where it is converted, so the epilogue needs only a few vector registers.
     {
-      const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * 2;
-      const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * 2u : 0u;
+      constexpr int CE = ACC_F32 ? 4 : 2;   // bytes per element of c
+      const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * CE;
+      const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * (uint32_t)CE : 0u;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
       auto take4 = [&](int i, int j, int q) {
         bf16x4 o;
@@ -791,7 +795,38 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
         }
         return __builtin_bit_cast(u32x2, o);
       };
-      if constexpr (Cfg::STAGED_EPILOGUE) {
+      if constexpr (ACC_F32) {
+        // c += product in fp32.  The 4 consecutive columns a lane holds are 16 bytes of c:
+        // read them, add, write them back; lanes l and l + 32 cover 32 contiguous bytes of a
+        // row, four such instructions one 128-byte line.
+#pragma unroll
+        for (int i = 0; i < ML; ++i) {
+          const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
+#pragma unroll
+          for (int j = 0; j < NB; ++j) {
+            uint32_t off[4];
+            u32x4 old[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+              off[q] = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 4u : kOutOfRange;
+              old[q] = __builtin_amdgcn_raw_buffer_load_b128(rc, off[q], 0, 0);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              f32x4 sum = __builtin_bit_cast(f32x4, old[q]);
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float v;
+                asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
+                sum[r] += v;
+              }
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum), rc, off[q], 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      } else if constexpr (Cfg::STAGED_EPILOGUE) {
         // Through a strip of LDS private to the wave: 32 rows x 64 columns go in as the
         // 8-byte pieces the lanes hold and come out as 16 bytes per lane, 8 lanes per row, so
         // that one store instruction writes 8 complete 128-byte lines.

@@ -105,6 +105,27 @@ void GroupedGemm(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tenso
   TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
 }
 
+// c (num_experts, hidden_in, hidden_out) fp32 += per expert a_e^T @ b_e; see gg_gmm_bf16_acc_f32.
+void AccumulateWeightGradient(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes) {
+  TORCH_CHECK(c.scalar_type() == torch::kFloat32, "grouped_gemm: the accumulated gradient must be float32");
+  // every other check is the one of the bf16 weight-gradient call
+  torch::Tensor shape_of_c = torch::empty(c.sizes(), torch::dtype(torch::kBFloat16).device(torch::kMeta));
+  Validate(a, b, shape_of_c, batch_sizes, /*trans_a=*/true, /*trans_b=*/false, /*on_device=*/false);
+  TORCH_CHECK(a.is_cuda() && b.is_cuda() && c.is_cuda(), "grouped_gemm: a, b and c must be GPU tensors");
+  TORCH_CHECK(b.device() == a.device() && c.device() == a.device(),
+              "grouped_gemm: a, b and c must be on the same GPU");
+  TORCH_CHECK(c.is_contiguous(), "grouped_gemm: c must be contiguous");
+  if (batch_sizes.is_cuda())
+    TORCH_CHECK(batch_sizes.device() == a.device(), "grouped_gemm: batch_sizes is on another GPU");
+  torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
+  const int rc = gg_gmm_bf16_acc_f32(a.data_ptr(), b.data_ptr(), c.data_ptr<float>(),
+                                     sizes.data_ptr<int64_t>(), sizes.is_cuda() ? 1 : 0, sizes.size(0),
+                                     a.size(0), a.size(1), b.size(1), static_cast<void*>(stream));
+  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+}
+
 // The on-device scheduler's view of the groups, as an int64 tensor
 // (num_experts, GG_SCHED_COLS) on `device`; see gg_debug_schedule.
 torch::Tensor DebugSchedule(torch::Tensor batch_sizes, int64_t tokens, int64_t hidden_in,
@@ -130,6 +151,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         [](torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes, bool trans_a,
            bool trans_b) { Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/false); },
         "Shape, rank and dtype checks of gmm without the device checks.");
+  m.def("accumulate_weight_gradient", &AccumulateWeightGradient,
+        "c (fp32) += per expert a_e^T @ b_e.");
   m.def("debug_schedule", &DebugSchedule, "Per-group table derived by the on-device scheduler.");
   m.attr("max_groups_per_launch") = GG_MAX_GROUPS_PER_LAUNCH;
   m.attr("sched_cols") = GG_SCHED_COLS;

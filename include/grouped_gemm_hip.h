@@ -69,6 +69,22 @@ int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_size
                 void* stream);
 
 /*
+ * Weight gradient accumulated in fp32: c[e] += a[S_e : S_e+m_e, :]^T @ b[S_e : S_e+m_e, :] for
+ * every group, the trans_a layout of gg_gmm_bf16 with an fp32 output that is added to instead of
+ * a bf16 output that is overwritten (alpha = 1, beta = 1).  a (tokens, hidden_in) and
+ * b (tokens, hidden_out) bf16, c (num_groups, hidden_in, hidden_out) fp32, all row-major and
+ * contiguous; c[e] of an empty group is left as it is.
+ *
+ * No counterpart in the reference, whose kernels fix alpha = 1, beta = 0 and a bf16 output
+ * (csrc/grouped_gemm.cu:255-257, 469); for trainers that keep fp32 main gradients and would
+ * otherwise run a second pass over c to add the bf16 result to them.
+ * Limits as for gg_gmm_bf16, with hidden_in and hidden_out below 2^20.
+ */
+int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* batch_sizes,
+                        int batch_sizes_on_device, int64_t num_groups, int64_t tokens,
+                        int64_t hidden_in, int64_t hidden_out, void* stream);
+
+/*
  * Runs only the on-device scheduler of gg_gmm_bf16 (same device code, same
  * arguments) and writes what it derived to `table_out`, a device buffer of
  * num_groups * GG_SCHED_COLS int64: per group the problem (m, n, k), leading

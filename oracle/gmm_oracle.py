@@ -121,6 +121,13 @@ def gmm_loop(a, b, batch_sizes, trans_a=False, trans_b=False, dtype=torch.float3
     return out
 
 
+def accumulate_weight_gradient_loop(a, b, batch_sizes, c0, dtype=torch.float64):
+    """c0[e] + a_e.t() @ b_e per expert: the accumulating form of the trans_a loop above.  The
+    product is the same loop (pinned as gmm_loop is), the accumulation an exact addition in
+    `dtype`; an empty expert leaves c0[e] as it is."""
+    return c0.to(dtype) + gmm_loop(a, b, batch_sizes, trans_a=True, dtype=dtype)
+
+
 def gmm_autograd_loop(a, b, batch_sizes, trans_b, grad, dtype=torch.float32):
     """Forward and both gradients by torch.autograd through the loop, on cloned fp32
     leaves, as the reference tests do (ops_test.py:67-80)."""

@@ -588,6 +588,61 @@ def test_traceable_operator_under_torch_compile(ops, trans_b):
         assert torch.equal(x, y)
 
 
+# ------------------------------------------------- fp32-accumulated weight gradient
+
+@pytest.mark.parametrize("on_device", [False, True])
+@pytest.mark.parametrize("sizes,hin,hout", [
+    ([128] * 8, 128, 128),
+    ([300, 0, 17, 1000, 0, 129], 520, 776),        # empty experts, ragged depth and width
+    ([0, 0, 0], 64, 72),
+    ([5] * 70, 264, 136),
+])
+def test_accumulated_weight_gradient(ops, oracle, sizes, hin, hout, on_device):
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    t = int(bs.sum())
+    g = torch.Generator().manual_seed(31)
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+    c0 = torch.randn(len(sizes), hin, hout, generator=g) * 8
+    _announce("accumulate", sizes, hin, hout, on_device)
+    c = c0.clone().cuda()
+    dev_bs = bs.cuda() if on_device else bs
+    got = ops.backend.accumulate_weight_gradient(a.cuda(), b.cuda(), dev_bs, c)
+    assert got is c
+    want = oracle.accumulate_weight_gradient_loop(a, b, bs, c0)
+    # fp32 accumulation of exact bf16 products: the only error is the order of fp32 sums
+    depth = max(sizes) if sizes else 0
+    tol = 1e-6 * (depth ** 0.5 + 4) * (want.abs().max().item() + 8 * depth ** 0.5 + 1)
+    assert (c.double().cpu() - want).abs().max().item() <= tol
+    for e, size in enumerate(sizes):                   # an empty expert's slice is untouched
+        if size == 0:
+            assert torch.equal(c[e].cpu(), c0[e])
+    # a second call adds the same product again: (c - c0) doubles, up to fp32 rounding
+    first = c.double().cpu() - c0.double()
+    ops.backend.accumulate_weight_gradient(a.cuda(), b.cuda(), dev_bs, c)
+    second = c.double().cpu() - c0.double()
+    assert (second - 2 * first).abs().max().item() <= 4 * tol
+
+
+def test_accumulated_weight_gradient_full_size_and_errors(ops, oracle):
+    from grouped_gemm_amd import workloads
+    w = workloads.make(4, device="cuda")                # 8 x 4096 rows, 4096 x 14336
+    sd = w.batch_sizes.cuda()
+    c = torch.zeros(8, w.hidden_in, w.hidden_out, device="cuda")
+    ops.backend.accumulate_weight_gradient(w.a, w.grad, sd, c)
+    bf16 = ops.backend.gmm(w.a, w.grad, sd, trans_a=True)
+    # same products, same fp32 accumulation order: rounding the fp32 result gives the bf16 one
+    assert torch.equal(c.to(torch.bfloat16), bf16)
+    ops.backend.accumulate_weight_gradient(w.a, w.grad, sd, c)
+    assert torch.equal(c.to(torch.bfloat16), (2 * bf16.float()).to(torch.bfloat16))
+    with pytest.raises(RuntimeError, match="float32"):
+        ops.backend.accumulate_weight_gradient(w.a, w.grad, sd, c.to(torch.bfloat16))
+    with pytest.raises(RuntimeError):
+        ops.backend.accumulate_weight_gradient(w.a, w.grad, sd, c[:, :, :-8].contiguous())
+    with pytest.raises(RuntimeError):
+        ops.backend.accumulate_weight_gradient(w.a, w.grad[:-1], sd, c)
+
+
 # ------------------------------------------------------------------------ edge cases
 
 def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):
