@@ -93,6 +93,10 @@ def main():
     ap.add_argument("--zeros", action="store_true",
                     help="diagnostic: all-zero inputs (no data toggling), to separate the power "
                          "limit from the kernel's cycle efficiency; not a valid benchmark result")
+    ap.add_argument("--vendor-loop", action="store_true",
+                    help="also time the reference's default algorithm on this GPU: one vendor GEMM "
+                         "(torch.matmul) per expert with host-resident sizes, for the workload's "
+                         "NN launch only (csrc/grouped_gemm.cu:396-413); adds a 'vendor_loop' object")
     ap.add_argument("--copy-bytes", type=int, default=0,
                     help="only run a plain device copy of this many bytes, 5 times (a known "
                          "traffic to scale the FETCH_SIZE / WRITE_SIZE counters by)")
@@ -203,6 +207,35 @@ def main():
                 } for n, ms in kernel_ms.items()},
         },
     }
+    if args.vendor_loop:
+        # the NN launch of this workload: forward, or the input gradient when b is stored transposed
+        which = "agrad" if w.trans_b else "fwd"
+        lhs_nn = w.grad if w.trans_b else w.a
+        sizes_host = w.batch_sizes.tolist()
+        res = torch.empty(lhs_nn.shape[0], w.b.shape[2], dtype=torch.bfloat16, device="cuda")
+
+        def loop():
+            start = 0
+            for e, m in enumerate(sizes_host):
+                if m:
+                    torch.matmul(lhs_nn[start:start + m], w.b[e], out=res[start:start + m])
+                start += m
+
+        for _ in range(3):
+            loop()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = max(3, min(args.steps, 20))
+        e0.record()
+        for _ in range(reps):
+            loop()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        out["vendor_loop"] = {"launch": f"NN ({which})", "experts": len(sizes_host), "ms": round(ms, 4),
+                              "TFLOP/s": round(flops_gemm / (ms * 1e-3) / 1e12, 2),
+                              "this_library_ms": round(kernel_ms[which], 4),
+                              "speedup": round(ms / kernel_ms[which], 3)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(out))
