@@ -5,14 +5,17 @@
 //
 // Every workgroup first derives the same schedule from batch_sizes (prefix sums of
 // rows and of tiles, kept in LDS), then walks tiles t = id, id + grid, ... .  A tile is
-// BM x BN outputs of one group.  Operand tiles go from HBM straight into LDS
+// up to BM x BN outputs of one group: a group's rows are split evenly over its tile rows,
+// and a tile issues MFMAs only for the 32-row blocks that have rows.  Operand tiles go from
+// HBM straight into LDS
 // (buffer_load_dwordx4 ... lds, 16 bytes per lane), through a ring of STAGES buffers;
 // rows past a group's end are cut off by the buffer descriptor's size, so they
 // arrive as zeros and no lane ever touches memory outside its group.  Fragments are read
 // from LDS with ds_read_b128 where the depth dimension is contiguous in memory and
 // with the transposing ds_read_b64_tr_b16 where it is not, feed
 // v_mfma_f32_32x32x16_bf16 with fp32 accumulators, and leave as bf16 through
-// buffer stores that the descriptor clips at the group's last row.
+// buffer stores that the descriptor clips at the group's last row (or are added to an fp32
+// output, in the accumulating form of the weight-gradient layout).
 #pragma once
 
 #include <hip/hip_runtime.h>
