@@ -93,6 +93,9 @@ def main():
     ap.add_argument("--zeros", action="store_true",
                     help="diagnostic: all-zero inputs (no data toggling), to separate the power "
                          "limit from the kernel's cycle efficiency; not a valid benchmark result")
+    ap.add_argument("--accumulate", action="store_true",
+                    help="time only the weight gradient in its accumulating form: c (fp32) += a^T b "
+                         "(backend.accumulate_weight_gradient) instead of the bf16 launch")
     ap.add_argument("--vendor-loop", action="store_true",
                     help="also time the reference's default algorithm on this GPU: one vendor GEMM "
                          "(torch.matmul) per expert with host-resident sizes, for the workload's "
@@ -130,7 +133,12 @@ def main():
         "bgrad": lambda: backend.gmm(lhs, rhs, sizes_dev, trans_a=True),
     }
     names = [n for n in ("fwd", "agrad", "bgrad") if n in w.gemms]
-    layout = {"fwd": "NT" if w.trans_b else "NN", "agrad": "NN" if w.trans_b else "NT", "bgrad": "TN"}
+    if args.accumulate:
+        main_grad = torch.zeros(w.batch_sizes.numel(), lhs.shape[1], rhs.shape[1], device="cuda")
+        calls["bgrad"] = lambda: backend.accumulate_weight_gradient(lhs, rhs, sizes_dev, main_grad)
+        names = ["bgrad"]
+    layout = {"fwd": "NT" if w.trans_b else "NN", "agrad": "NN" if w.trans_b else "NT",
+              "bgrad": "TN, fp32 +=" if args.accumulate else "TN"}
 
     def step(events=None):
         for n in names:
@@ -156,6 +164,8 @@ def main():
 
     flops_gemm = w.flops_per_gemm()
     bytes_gemm = w.bytes_per_gemm()
+    if args.accumulate:   # the fp32 output is read and written: 8 bytes per element instead of 2
+        bytes_gemm += 6 * w.batch_sizes.numel() * w.hidden_in * w.hidden_out
     ms_per_step = elapsed / args.steps * 1e3
     value = flops_gemm * len(names) / (ms_per_step * 1e-3) / 1e12
     samples = {n: sorted(a.elapsed_time(b) for a, b in ev) for n, ev in events.items()}
@@ -164,7 +174,8 @@ def main():
     achieved = flops_gemm / (kernel_ms[slowest] * 1e-3) / 1e12
 
     out = {
-        "metric": "bf16 grouped-GEMM TFLOP/s, Mixtral-8x7B w1 shape fwd+bwd",
+        "metric": ("bf16 grouped-GEMM TFLOP/s, weight gradient accumulated into fp32" if args.accumulate
+                   else "bf16 grouped-GEMM TFLOP/s, Mixtral-8x7B w1 shape fwd+bwd"),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
