@@ -801,33 +801,37 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
       if constexpr (ACC_F32) {
         // c += product in fp32.  The 4 consecutive columns a lane holds are 16 bytes of c:
         // read them, add, write them back; lanes l and l + 32 cover 32 contiguous bytes of a
-        // row, four such instructions one 128-byte line.
+        // row, four such instructions one 128-byte line.  All reads of a 32-row block row are
+        // issued before the first addition: 16 in flight per lane measured faster than a
+        // rolling 8 + 8.
 #pragma unroll
         for (int i = 0; i < ML; ++i) {
           const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
+          uint32_t off[NB][4];
+          u32x4 old[NB][4];
 #pragma unroll
-          for (int j = 0; j < NB; ++j) {
-            uint32_t off[4];
-            u32x4 old[4];
+          for (int j = 0; j < NB; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
-              off[q] = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 4u : kOutOfRange;
-              old[q] = __builtin_amdgcn_raw_buffer_load_b128(rc, off[q], 0, 0);
+              off[j][q] = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 4u : kOutOfRange;
+              old[j][q] = __builtin_amdgcn_raw_buffer_load_b128(rc, off[j][q], 0, 0);
             }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = 0; j < NB; ++j)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              f32x4 sum = __builtin_bit_cast(f32x4, old[q]);
+              f32x4 sum = __builtin_bit_cast(f32x4, old[j][q]);
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
                 float v;
                 asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
                 sum[r] += v;
               }
-              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum), rc, off[q], 0, 0);
+              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum), rc, off[j][q], 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       } else if constexpr (Cfg::STAGED_EPILOGUE) {
         // Through a strip of LDS private to the wave: 32 rows x 64 columns go in as the
