@@ -643,6 +643,36 @@ def test_accumulated_weight_gradient_full_size_and_errors(ops, oracle):
         ops.backend.accumulate_weight_gradient(w.a, w.grad[:-1], sd, c)
 
 
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+@pytest.mark.parametrize("long_side", ["in", "out"])
+def test_hidden_sizes_at_the_documented_limit(ops, oracle, layout, long_side):
+    # hidden_in or hidden_out = 2**22 - 8, the largest allowed: the 32-bit byte offsets inside a
+    # tile (row * leading dimension) are then at their largest
+    trans_a, trans_b = layout
+    big, small = (1 << 22) - 8, 8
+    hin, hout = (big, small) if long_side == "in" else (small, big)
+    sizes = [3, 0, 6]
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    t = int(bs.sum())
+    g = torch.Generator().manual_seed(37)
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    if trans_a:
+        b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+    else:
+        b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+    _announce("limit", layout, hin, hout)
+    out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda(), trans_a=trans_a, trans_b=trans_b)
+    want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
+    # a depth of four million: compare with a tolerance that grows like sqrt(depth)
+    scale = max(1.0, (hin if not trans_a else max(sizes)) ** 0.5 / 64)
+    err = (out.float().cpu() - want).abs()
+    assert bool((err <= scale * (ATOL + RTOL * want.abs())).all()), err.max().item()
+    with pytest.raises(RuntimeError, match="2\\^22"):
+        too_big = torch.zeros(1, (1 << 22), dtype=torch.bfloat16, device="cuda")
+        ops.backend.gmm(too_big, torch.zeros(1, (1 << 22), 8, dtype=torch.bfloat16, device="cuda"),
+                        torch.tensor([1]))
+
+
 # ------------------------------------------------------------------------ edge cases
 
 def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):
