@@ -145,6 +145,10 @@ def test_c_abi_argument_errors_need_no_device():
     misaligned = lib.gg_gmm_bf16(ptr(4096), ptr(8192 + 2), ptr(12288), sizes, 0, i64(2), i64(8), i64(16),
                                  i64(24), 0, 0, None)
     assert misaligned == -2 and b"16-byte aligned" in lib.gg_last_error()
+    # the accumulating form: tighter limit on the hidden sizes, checked before anything else
+    acc = lib.gg_gmm_bf16_acc_f32(ptr(4096), ptr(8192), ptr(12288), sizes, 0, i64(2), i64(8), i64(1 << 20),
+                                  i64(24), None)
+    assert acc == -2 and b"2^20" in lib.gg_last_error()
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     assert lib.gg_tile_shape(i64(8), i64(32768), 0, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
     assert (bm.value, bn.value, bk.value) == (256, 256, 64)
