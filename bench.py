@@ -8,7 +8,8 @@ exactly the calls grouped_gemm.ops.GroupedGemm makes: forward (NN), input gradie
 timed region.  Prints ONE JSON line.
 
   value      TFLOP/s over the timed steps (2*T*K*N flops per GEMM, padding never counted)
-  roofline   the slowest of the three kernels against the bf16 dense MFMA peak, its
+  roofline   the slowest of the three kernels against the roof that bounds the workload (bf16
+             dense MFMA peak, or the HBM peak when flops / algorithmic bytes is below the ridge), its
              duration taken from HIP events recorded around each launch inside the timed
              region (same stream the kernels run on)
   cpu_baseline  the oracle's per-expert loop (bf16 CPU tensors, torch CPU matmul) on a
@@ -171,7 +172,12 @@ def main():
     samples = {n: sorted(a.elapsed_time(b) for a, b in ev) for n, ev in events.items()}
     kernel_ms = {n: sum(v) / len(v) for n, v in samples.items()}
     slowest = max(kernel_ms, key=kernel_ms.get)
-    achieved = flops_gemm / (kernel_ms[slowest] * 1e-3) / 1e12
+    # which roof bounds the workload: arithmetic intensity against the ridge of the two peaks
+    hbm_bound = flops_gemm / bytes_gemm < PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)
+    if hbm_bound:
+        achieved, peak, unit = bytes_gemm / (kernel_ms[slowest] * 1e-3) / 1e9, PEAK_HBM_GBPS, "GB/s"
+    else:
+        achieved, peak, unit = flops_gemm / (kernel_ms[slowest] * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
 
     out = {
         "metric": ("bf16 grouped-GEMM TFLOP/s, weight gradient accumulated into fp32" if args.accumulate
@@ -195,12 +201,12 @@ def main():
         },
         "frac_of_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
         "roofline": {
-            "bound": "mfma",
+            "bound": "hbm" if hbm_bound else "mfma",
             "kernel": f"gmm_kernel {layout[slowest]} ({slowest})",
             "achieved": round(achieved, 2),
-            "peak": PEAK_BF16_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+            "peak": peak,
+            "unit": unit,
+            "frac": round(achieved / peak, 4),
             "traffic": (round(MEASURED_TRAFFIC_BYTES[args.config][slowest])
                         if args.config in MEASURED_TRAFFIC_BYTES and not args.zeros else None),
             "algorithmic_bytes": bytes_gemm,
