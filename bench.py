@@ -30,10 +30,13 @@ PEAK_HBM_GBPS = 8000.0
 
 # Bytes per launch between L2 and the fabric for the default workload, from two rocprofv3 --pmc
 # runs of this file (FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by a 1 GiB device copy, both in
-# KiB); the figures and commands are in profiles/gmm_kernel_mixtral_w1_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES = {
-    2: {"fwd": (4458000 * 2.0 + 917600) * 1024, "agrad": (3812000 * 2.0 + 262144) * 1024,
-        "bgrad": (2755000 * 2.0 + 917500) * 1024},
+# KiB).  Profiled once, not in this run: `source` names the summary under profiles/ that holds the
+# figures, the commands and the revision of the kernel they were taken on.
+_TRAFFIC_SOURCE = "profiles/gmm_kernel_mixtral_w1_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiled once)"
+MEASURED_TRAFFIC = {
+    2: {"fwd": {"bytes": (4458000 * 2.0 + 917600) * 1024, "source": _TRAFFIC_SOURCE},
+        "agrad": {"bytes": (3812000 * 2.0 + 262144) * 1024, "source": _TRAFFIC_SOURCE},
+        "bgrad": {"bytes": (2755000 * 2.0 + 917500) * 1024, "source": _TRAFFIC_SOURCE}},
 }
 
 
@@ -84,6 +87,113 @@ def cpu_baseline(w, budget_s=12.0):
                       f"(torch CPU bf16 matmul, {cores} threads), {t:.1f} s"}
 
 
+WORKLOAD_NAMES = {
+    2: ("bf16 grouped-GEMM TFLOP/s, Mixtral-8x7B w1 shape fwd+bwd",
+        "forward + input-gradient + weight-gradient grouped GEMMs"),
+    3: ("bf16 grouped-GEMM TFLOP/s, ragged fine-grained MoE forward", "forward grouped GEMM"),
+    4: ("bf16 grouped-GEMM TFLOP/s, weight gradient (trans_a) alone", "weight-gradient grouped GEMM"),
+    5: ("bf16 grouped-GEMM TFLOP/s, DeepSeek-V3-style expert share fwd+bwd",
+        "forward + input-gradient + weight-gradient grouped GEMMs (b stored transposed)"),
+}
+
+
+def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0):
+    """Times the grouped GEMMs of one configuration; returns (workload, names, layout, ms_per_step,
+    per-launch samples in ms)."""
+    import torch
+    from grouped_gemm import backend
+    from grouped_gemm_amd import workloads
+
+    w = workloads.make(config, device="cuda")
+    if zeros:
+        w.a.zero_(), w.b.zero_(), w.grad.zero_()
+    sizes_dev = w.batch_sizes.cuda()
+    lhs, rhs = (w.grad, w.a) if w.trans_b else (w.a, w.grad)
+
+    def gmm(a, b, trans_a=False, trans_b=False):
+        if not flags:
+            return backend.gmm(a, b, sizes_dev, trans_a=trans_a, trans_b=trans_b)
+        c = backend._allocate_output(a, b, sizes_dev, trans_a, trans_b)
+        backend.backend.gmm_with_flags(a, b, c, sizes_dev, trans_a, trans_b, flags)
+        return c
+
+    calls = {
+        "fwd": lambda: gmm(w.a, w.b, trans_b=w.trans_b),
+        "agrad": lambda: gmm(w.grad, w.b, trans_b=not w.trans_b),
+        "bgrad": lambda: gmm(lhs, rhs, trans_a=True),
+    }
+    names = [n for n in ("fwd", "agrad", "bgrad") if n in w.gemms]
+    if accumulate:
+        main_grad = torch.zeros(w.batch_sizes.numel(), lhs.shape[1], rhs.shape[1], device="cuda")
+        calls["bgrad"] = lambda: backend.accumulate_weight_gradient(lhs, rhs, sizes_dev, main_grad)
+        names = ["bgrad"]
+    layout = {"fwd": "NT" if w.trans_b else "NN", "agrad": "NN" if w.trans_b else "NT",
+              "bgrad": "TN, fp32 +=" if accumulate else "TN"}
+
+    def step(events=None):
+        for n in names:
+            if events is not None:
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                calls[n]()
+                e1.record()
+                events[n].append((e0, e1))
+            else:
+                calls[n]()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    events = {n: [] for n in names}
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(events)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) / steps * 1e3
+    samples = {n: sorted(a.elapsed_time(b) for a, b in ev) for n, ev in events.items()}
+    return w, names, layout, ms_per_step, samples
+
+
+def summarize(w, names, layout, ms_per_step, samples, accumulate=False):
+    """value, roofline object and per-kernel table of one timed workload."""
+    flops_gemm = w.flops_per_gemm()
+    bytes_gemm = w.bytes_per_gemm()
+    if accumulate:   # the fp32 output is read and written: 8 bytes per element instead of 2
+        bytes_gemm += 6 * w.batch_sizes.numel() * w.hidden_in * w.hidden_out
+    value = flops_gemm * len(names) / (ms_per_step * 1e-3) / 1e12
+    kernel_ms = {n: sum(v) / len(v) for n, v in samples.items()}
+    slowest = max(kernel_ms, key=kernel_ms.get)
+    # which roof bounds the workload: arithmetic intensity against the ridge of the two peaks
+    hbm_bound = flops_gemm / bytes_gemm < PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)
+    if hbm_bound:
+        achieved, peak, unit = bytes_gemm / (kernel_ms[slowest] * 1e-3) / 1e9, PEAK_HBM_GBPS, "GB/s"
+    else:
+        achieved, peak, unit = flops_gemm / (kernel_ms[slowest] * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
+    roofline = {
+        "bound": "hbm" if hbm_bound else "mfma",
+        "kernel": f"gmm_kernel {layout[slowest]} ({slowest})",
+        "achieved": round(achieved, 2),
+        "peak": peak,
+        "unit": unit,
+        "frac": round(achieved / peak, 4),
+        "algorithmic_bytes": bytes_gemm,
+        "launch_ms": round(kernel_ms[slowest], 4),
+        "flops_per_launch": flops_gemm,
+        "per_kernel": {
+            f"{layout[n]} ({n})": {
+                "ms": round(ms, 4),
+                "median_ms": round(samples[n][len(samples[n]) // 2], 4),
+                "min_ms": round(samples[n][0], 4),
+                "TFLOP/s": round(flops_gemm / (ms * 1e-3) / 1e12, 2),
+                "frac_mfma": round(flops_gemm / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
+                "GB/s": round(bytes_gemm / (ms * 1e-3) / 1e9, 1),
+                "frac_hbm": round(bytes_gemm / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
+            } for n, ms in kernel_ms.items()},
+    }
+    return value, roofline, slowest, kernel_ms
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -91,9 +201,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration (2 = Mixtral w1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of the other configurations that the default run appends")
     ap.add_argument("--zeros", action="store_true",
                     help="diagnostic: all-zero inputs (no data toggling), to separate the power "
                          "limit from the kernel's cycle efficiency; not a valid benchmark result")
+    ap.add_argument("--flags", type=int, default=0,
+                    help="diagnostic: GG_FLAG_* scheduling switches of include/grouped_gemm_hip.h "
+                         "(1 whole tiles, 2 one tile class, 4 row pieces); results are unchanged")
     ap.add_argument("--accumulate", action="store_true",
                     help="time only the weight gradient in its accumulating form: c (fp32) += a^T b "
                          "(backend.accumulate_weight_gradient) instead of the bf16 launch")
@@ -110,8 +225,6 @@ def main():
                  "needs no exchange inside this operator and is left to the caller. Use --gpus 1.")
 
     import torch
-    from grouped_gemm import backend
-    from grouped_gemm_amd import workloads
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
@@ -123,65 +236,20 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copied_bytes": args.copy_bytes, "times": 5}))
         return
-    w = workloads.make(args.config, device="cuda")
-    if args.zeros:
-        w.a.zero_(), w.b.zero_(), w.grad.zero_()
-    sizes_dev = w.batch_sizes.cuda()
-    lhs, rhs = (w.grad, w.a) if w.trans_b else (w.a, w.grad)
-    calls = {
-        "fwd": lambda: backend.gmm(w.a, w.b, sizes_dev, trans_b=w.trans_b),
-        "agrad": lambda: backend.gmm(w.grad, w.b, sizes_dev, trans_b=not w.trans_b),
-        "bgrad": lambda: backend.gmm(lhs, rhs, sizes_dev, trans_a=True),
-    }
-    names = [n for n in ("fwd", "agrad", "bgrad") if n in w.gemms]
-    if args.accumulate:
-        main_grad = torch.zeros(w.batch_sizes.numel(), lhs.shape[1], rhs.shape[1], device="cuda")
-        calls["bgrad"] = lambda: backend.accumulate_weight_gradient(lhs, rhs, sizes_dev, main_grad)
-        names = ["bgrad"]
-    layout = {"fwd": "NT" if w.trans_b else "NN", "agrad": "NN" if w.trans_b else "NT",
-              "bgrad": "TN, fp32 +=" if args.accumulate else "TN"}
-
-    def step(events=None):
-        for n in names:
-            if events is not None:
-                e0 = torch.cuda.Event(enable_timing=True)
-                e1 = torch.cuda.Event(enable_timing=True)
-                e0.record()
-                calls[n]()
-                e1.record()
-                events[n].append((e0, e1))
-            else:
-                calls[n]()
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    events = {n: [] for n in names}
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(events)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-
+    w, names, layout, ms_per_step, samples = run_workload(args.config, args.steps, args.warmup,
+                                                          args.accumulate, args.zeros, args.flags)
+    value, roofline, slowest, kernel_ms = summarize(w, names, layout, ms_per_step, samples, args.accumulate)
     flops_gemm = w.flops_per_gemm()
-    bytes_gemm = w.bytes_per_gemm()
-    if args.accumulate:   # the fp32 output is read and written: 8 bytes per element instead of 2
-        bytes_gemm += 6 * w.batch_sizes.numel() * w.hidden_in * w.hidden_out
-    ms_per_step = elapsed / args.steps * 1e3
-    value = flops_gemm * len(names) / (ms_per_step * 1e-3) / 1e12
-    samples = {n: sorted(a.elapsed_time(b) for a, b in ev) for n, ev in events.items()}
-    kernel_ms = {n: sum(v) / len(v) for n, v in samples.items()}
-    slowest = max(kernel_ms, key=kernel_ms.get)
-    # which roof bounds the workload: arithmetic intensity against the ridge of the two peaks
-    hbm_bound = flops_gemm / bytes_gemm < PEAK_BF16_TFLOPS * 1e12 / (PEAK_HBM_GBPS * 1e9)
-    if hbm_bound:
-        achieved, peak, unit = bytes_gemm / (kernel_ms[slowest] * 1e-3) / 1e9, PEAK_HBM_GBPS, "GB/s"
-    else:
-        achieved, peak, unit = flops_gemm / (kernel_ms[slowest] * 1e-3) / 1e12, PEAK_BF16_TFLOPS, "TFLOP/s"
+    traffic = MEASURED_TRAFFIC.get(args.config, {}).get(slowest) if not (args.zeros or args.accumulate or args.flags) else None
+    roofline["traffic"] = round(traffic["bytes"]) if traffic else None
+    roofline["traffic_source"] = traffic["source"] if traffic else None
+    metric, what = WORKLOAD_NAMES[args.config]
+    if args.accumulate:
+        metric, what = ("bf16 grouped-GEMM TFLOP/s, weight gradient accumulated into fp32",
+                        "weight-gradient grouped GEMM added to an fp32 output")
 
     out = {
-        "metric": ("bf16 grouped-GEMM TFLOP/s, weight gradient accumulated into fp32" if args.accumulate
-                   else "bf16 grouped-GEMM TFLOP/s, Mixtral-8x7B w1 shape fwd+bwd"),
+        "metric": metric,
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "n_gpus": 1,
@@ -195,35 +263,15 @@ def main():
         "data": "zeros (diagnostic, not a benchmark result)" if args.zeros else "synthetic",
         "config": {
             "workload": f"configs[{args.config - 1}]: {w.batch_sizes.numel()} experts, {w.tokens} routed rows, "
-                        f"{w.hidden_in}x{w.hidden_out}, forward + input-gradient + weight-gradient grouped GEMMs",
+                        f"{w.hidden_in}x{w.hidden_out}, {what}",
             "batch_sizes": w.batch_sizes.tolist() if w.batch_sizes.numel() <= 16 else "see workloads.make",
             "batch_sizes_on_device": True,
         },
         "frac_of_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
-        "roofline": {
-            "bound": "hbm" if hbm_bound else "mfma",
-            "kernel": f"gmm_kernel {layout[slowest]} ({slowest})",
-            "achieved": round(achieved, 2),
-            "peak": peak,
-            "unit": unit,
-            "frac": round(achieved / peak, 4),
-            "traffic": (round(MEASURED_TRAFFIC_BYTES[args.config][slowest])
-                        if args.config in MEASURED_TRAFFIC_BYTES and not args.zeros else None),
-            "algorithmic_bytes": bytes_gemm,
-            "launch_ms": round(kernel_ms[slowest], 4),
-            "flops_per_launch": flops_gemm,
-            "per_kernel": {
-                f"{layout[n]} ({n})": {
-                    "ms": round(ms, 4),
-                    "median_ms": round(samples[n][len(samples[n]) // 2], 4),
-                    "min_ms": round(samples[n][0], 4),
-                    "TFLOP/s": round(flops_gemm / (ms * 1e-3) / 1e12, 2),
-                    "frac_mfma": round(flops_gemm / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4),
-                    "GB/s": round(bytes_gemm / (ms * 1e-3) / 1e9, 1),
-                    "frac_hbm": round(bytes_gemm / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4),
-                } for n, ms in kernel_ms.items()},
-        },
+        "roofline": roofline,
     }
+    if args.flags:
+        out["config"]["diagnostic_flags"] = args.flags
     if args.vendor_loop:
         # the NN launch of this workload: forward, or the input gradient when b is stored transposed
         which = "agrad" if w.trans_b else "fwd"
@@ -255,6 +303,26 @@ def main():
                               "speedup": round(ms / kernel_ms[which], 3)}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
+    # The other measured configurations, shortly, so that one default run shows all of them.
+    default_run = not (args.no_other_configs or args.zeros or args.flags or args.accumulate or args.vendor_loop)
+    if default_run and args.config == 2:
+        del w
+        others = {}
+        for cfg, acc in ((3, False), (4, False), (4, True), (5, False)):
+            torch.cuda.empty_cache()
+            res = run_workload(cfg, min(args.steps, 10), min(args.warmup, 3), accumulate=acc)
+            v, roof, _, _ = summarize(*res, accumulate=acc)
+            others[f"configs[{cfg - 1}]" + (" accumulate" if acc else "")] = {
+                "workload": WORKLOAD_NAMES[cfg][1] if not acc else "weight gradient added to an fp32 output",
+                "experts": res[0].batch_sizes.numel(), "rows": res[0].tokens,
+                "hidden": f"{res[0].hidden_in}x{res[0].hidden_out}", "steps": min(args.steps, 10),
+                "ms_per_step": round(res[3], 4), "TFLOP/s": round(v, 2),
+                "bound": roof["bound"], "achieved": roof["achieved"], "unit": roof["unit"], "frac": roof["frac"],
+                "slowest_kernel": roof["kernel"],
+                "per_kernel_ms": {k: d["ms"] for k, d in roof["per_kernel"].items()},
+            }
+            del res
+        out["other_configs"] = others
     print(json.dumps(out))
 
 

@@ -5,12 +5,15 @@
 
 Usage: python grouped_gemm_amd/build.py [--force]
 hipcc cross-compiles gfx950 without a GPU, so this runs anywhere the ROCm toolchain
-and PyTorch-ROCm are installed.
+and PyTorch-ROCm are installed.  The kernel variants (csrc/gmm_variants.def) are compiled as
+separate translation units, several at a time; objects are kept under grouped_gemm_amd/build/.
 """
 import os
+import re
 import subprocess
 import sys
 import sysconfig
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -18,11 +21,15 @@ ROOT = os.path.dirname(HERE)
 HIP_LIB = os.path.join(HERE, "libgrouped_gemm_hip.so")
 EXT_LIB = os.path.join(HERE, "grouped_gemm_backend" + sysconfig.get_config_var("EXT_SUFFIX"))
 
+OBJ_DIR = os.path.join(HERE, "build")
+
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC",
     # packed fp32 instructions are switched off for device code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # the asm that loads into LDS names m0 as clobbered; clang notes that m0 is a reserved register
+    "-Wno-inline-asm",
 ]
 
 
@@ -33,24 +40,42 @@ def _newer(target, sources):
     return all(os.path.getmtime(s) <= t for s in sources)
 
 
-def _run(cmd):
-    print("+", " ".join(cmd), flush=True)
+def _run(cmd, quiet=False):
+    if not quiet:
+        print("+", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines()
                     if "is not a recognized feature for this target" not in l)
     if res.returncode != 0:
-        raise RuntimeError("build step failed:\n" + out)
+        raise RuntimeError("build step failed: " + " ".join(cmd) + "\n" + out)
     if out.strip():
         print(out)
 
 
-def build_hip(force=False):
-    sources = [os.path.join(CSRC, f) for f in ("gmm_api.hip", "gmm_kernel.hpp")]
-    sources.append(os.path.join(ROOT, "include", "grouped_gemm_hip.h"))
-    if not force and _newer(HIP_LIB, sources):
-        return HIP_LIB
+def variant_indices():
+    """Indices listed in csrc/gmm_variants.def: one translation unit per kernel variant."""
+    text = open(os.path.join(CSRC, "gmm_variants.def")).read()
+    return [int(m) for m in re.findall(r"^GG_VARIANT\((\d+),", text, flags=re.M)]
+
+
+def build_hip(force=False, jobs=None):
+    headers = [os.path.join(CSRC, f) for f in ("gmm_kernel.hpp", "gmm_variants.hpp", "gmm_variants.def")]
+    headers.append(os.path.join(ROOT, "include", "grouped_gemm_hip.h"))
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    _run([hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, "gmm_api.hip"), "-o", HIP_LIB])
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(OBJ_DIR, "gmm_api.o"), [])]
+    for i in variant_indices():
+        units.append((os.path.join(CSRC, "gmm_variant.hip"), os.path.join(OBJ_DIR, f"gmm_variant_{i}.o"),
+                      [f"-DGG_VARIANT_INDEX={i}"]))
+    todo = [u for u in units if force or not _newer(u[1], [u[0]] + headers)]
+    jobs = jobs or min(len(todo) or 1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1)))
+    if todo:
+        print(f"compiling {len(todo)} translation units with {hipcc}, {jobs} at a time", flush=True)
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            list(pool.map(lambda u: _run([hipcc] + HIPCC_FLAGS + u[2] + ["-c", u[0], "-o", u[1]], quiet=True), todo))
+    objects = [u[1] for u in units]
+    if todo or not _newer(HIP_LIB, objects):
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", HIP_LIB])
     return HIP_LIB
 
 

@@ -1,5 +1,5 @@
 // Host side of the C ABI declared in include/grouped_gemm_hip.h: argument checks,
-// kernel selection and the single launch.  No torch types, no allocation, no sync.
+// kernel selection and the launches.  No torch types, no allocation, no sync.
 #include "../../include/grouped_gemm_hip.h"
 
 #include <hip/hip_runtime.h>
@@ -10,9 +10,18 @@
 #include <cstring>
 #include <mutex>
 
-#include "gmm_kernel.hpp"
+#include "gmm_variants.hpp"
+
+namespace gg {
+#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_) const VariantOps* variant_ops_##index();
+#include "gmm_variants.def"
+#undef GG_VARIANT
+}  // namespace gg
 
 namespace {
+
+using gg::Short;
+using gg::Wide;
 
 thread_local char g_err[512] = "";
 
@@ -31,46 +40,36 @@ int fail(int code, const char* fmt, ...) {
       return fail(GG_EHIP, "%s failed: %s", #call, hipGetErrorString(err__));            \
   } while (0)
 
-// Tile shapes.  Wide: 256 x 256 outputs per workgroup, 2 x 2 waves of 128 x 128.  Short: 128 x 256,
-// 1 x 4 waves of 128 x 64, for calls whose groups average few rows: with at most 128 rows per
-// group all four waves then share the rows instead of two of them idling (measured 4-7 % faster
-// below about 100 rows per group, slower from 128 on).  The weight-gradient layout always uses the
-// wide shape: its ragged dimension is the depth, not the rows.
-#ifndef GG_GROUP_M
-#define GG_GROUP_M 4
-#endif
-// The weight-gradient layout with shallow groups is mostly output writes; there an odd band
-// height measures 5-8 % faster than 4 (the bands then do not line up with the 32-tile runs the
-// XCDs take, which spreads what is written at one time over more of the memory channels).
-#ifndef GG_GROUP_M_SHALLOW
-#define GG_GROUP_M_SHALLOW 3
-#endif
-#ifndef GG_SHALLOW_BELOW
-#define GG_SHALLOW_BELOW 1024   // average rows per group below which GG_GROUP_M_SHALLOW is used
-#endif
-#ifndef GG_SHORT_BELOW
-#define GG_SHORT_BELOW 112   // average rows per group below which the short shape is used
-#endif
-constexpr int BK = 64, STAGES = 2;
-struct Wide {
-  static constexpr int BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2;
+const gg::VariantOps* (*const kVariantGetters[])() = {
+#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_) &gg::variant_ops_##index,
+#include "gmm_variants.def"
+#undef GG_VARIANT
 };
-struct Short {
-  static constexpr int BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
-};
+constexpr int kNumVariants = sizeof(kVariantGetters) / sizeof(kVariantGetters[0]);
 
-// GG_TAIL_SPLIT=0 in the environment keeps the tiles of the last round whole (read at every call).
-int tail_split() {
-  const char* e = getenv("GG_TAIL_SPLIT");
-  return e != nullptr && e[0] == '0' ? 0 : 1;
+const gg::VariantOps* find_variant(int dt, int layout, int shape, int epilogue) {
+  for (int i = 0; i < kNumVariants; ++i) {
+    const gg::VariantOps* v = kVariantGetters[i]();
+    if (v->dt == dt && v->layout == layout && v->shape == shape && v->epilogue == epilogue) return v;
+  }
+  return nullptr;
 }
 
+// Tile rows per band of the in-group tile order.  The weight-gradient layout with shallow groups
+// is mostly output writes; there an odd band height measures 5-8 % faster than 4 (the bands then
+// do not line up with the 32-tile runs the XCDs take, which spreads what is written at one time
+// over more of the memory channels).
+constexpr int kBandHeight = 4;
+constexpr int kBandHeightShallow = 3;
+constexpr int kShallowBelow = 1024;   // average rows per group below which the shallow height is used
+constexpr int kShortBelow = 112;      // average rows per group below which the short tile shape is used
+
 int band_height(int64_t num_groups, int64_t tokens, int trans_a) {
-  return trans_a && tokens < (int64_t)GG_SHALLOW_BELOW * num_groups ? GG_GROUP_M_SHALLOW : GG_GROUP_M;
+  return trans_a && tokens < (int64_t)kShallowBelow * num_groups ? kBandHeightShallow : kBandHeight;
 }
 
 bool use_short_shape(int64_t num_groups, int64_t tokens, int trans_a) {
-  return !trans_a && num_groups > 0 && tokens < (int64_t)GG_SHORT_BELOW * num_groups;
+  return !trans_a && num_groups > 0 && tokens < (int64_t)kShortBelow * num_groups;
 }
 
 struct DeviceInfo {
@@ -78,6 +77,7 @@ struct DeviceInfo {
   bool ok = false;
 };
 
+// Per device, once: the architecture check and the LDS limit of every kernel variant.
 int device_info(DeviceInfo* out) {
   static DeviceInfo cache[64];
   static std::mutex mu;
@@ -90,6 +90,7 @@ int device_info(DeviceInfo* out) {
     GG_HIP(hipGetDeviceProperties(&prop, dev));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
       return fail(GG_EHIP, "this library is built for gfx950 only, device is %s", prop.gcnArchName);
+    for (int i = 0; i < kNumVariants; ++i) GG_HIP(kVariantGetters[i]()->prepare());
     cache[dev].cus = prop.multiProcessorCount;
     cache[dev].ok = true;
   }
@@ -97,76 +98,22 @@ int device_info(DeviceInfo* out) {
   return GG_OK;
 }
 
-template <typename S, int LAYOUT, bool HOST_SIZES, bool ACC_F32 = false>
-int launch(const gg::GmmParams& p, const gg::HostSizes* hs, int grid, hipStream_t stream) {
-  using Cfg = gg::GmmConfig<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N>;
-  constexpr int kThreads = S::WAVES_M * S::WAVES_N * 64;
-  const void* kernel = reinterpret_cast<const void*>(
-      &gg::gmm_kernel<LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, HOST_SIZES, ACC_F32>);
-  // raising the dynamic LDS limit is per device and per kernel; do it once each
-  static std::mutex mu;
-  static bool done[64] = {};
-  int dev = 0;
-  GG_HIP(hipGetDevice(&dev));
-  {
-    std::lock_guard<std::mutex> lock(mu);
-    if (!done[dev]) {
-      GG_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 Cfg::LDS_BYTES));
-      done[dev] = true;
-    }
-  }
-  gg::GmmParams params = p;
-  gg::HostSizes sizes_arg;
-  gg::NoSizes no_sizes;
-  void* args[2];
-  args[0] = &params;
-  if constexpr (HOST_SIZES) {
-    sizes_arg = *hs;
-    args[1] = &sizes_arg;
-  } else {
-    args[1] = &no_sizes;
-  }
-  GG_HIP(hipLaunchKernel(kernel, dim3(grid), dim3(kThreads), args, Cfg::LDS_BYTES, stream));
-  return GG_OK;
-}
-
-template <typename S, int LAYOUT, bool HOST_SIZES>
-int launch_dump(const gg::GmmParams& p, const gg::HostSizes* hs, hipStream_t stream) {
-  auto kernel = gg::schedule_dump_kernel<LAYOUT, S::BM, S::BN, HOST_SIZES>;
-  if constexpr (HOST_SIZES) {
-    hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, stream, p, *hs);
-  } else {
-    hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, stream, p, gg::NoSizes{});
-  }
+template <typename S, int LAYOUT>
+int launch_dump(const gg::GmmParams& p, const gg::HostSizes& hs, hipStream_t stream) {
+  hipLaunchKernelGGL((gg::schedule_dump_kernel<LAYOUT, S::BM, S::BN>), dim3(1), dim3(64), 0, stream, p, hs);
   GG_HIP(hipGetLastError());
   return GG_OK;
 }
 
-// out_f32: the accumulating form (weight-gradient layout only).
-template <bool HOST_SIZES>
-int dispatch(bool short_shape, int layout, bool out_f32, const gg::GmmParams& p, const gg::HostSizes* hs,
-             int grid, hipStream_t stream) {
-  if (out_f32) return launch<Wide, gg::kTN, HOST_SIZES, true>(p, hs, grid, stream);
-  if (layout == gg::kTN) return launch<Wide, gg::kTN, HOST_SIZES>(p, hs, grid, stream);
-  if (short_shape) {
-    return layout == gg::kNN ? launch<Short, gg::kNN, HOST_SIZES>(p, hs, grid, stream)
-                             : launch<Short, gg::kNT, HOST_SIZES>(p, hs, grid, stream);
-  }
-  return layout == gg::kNN ? launch<Wide, gg::kNN, HOST_SIZES>(p, hs, grid, stream)
-                           : launch<Wide, gg::kNT, HOST_SIZES>(p, hs, grid, stream);
-}
-
-template <bool HOST_SIZES>
-int dispatch_dump(bool short_shape, int layout, const gg::GmmParams& p, const gg::HostSizes* hs,
+int dispatch_dump(bool short_shape, int layout, const gg::GmmParams& p, const gg::HostSizes& hs,
                   hipStream_t stream) {
-  if (layout == gg::kTN) return launch_dump<Wide, gg::kTN, HOST_SIZES>(p, hs, stream);
+  if (layout == gg::kTN) return launch_dump<Wide, gg::kTN>(p, hs, stream);
   if (short_shape) {
-    return layout == gg::kNN ? launch_dump<Short, gg::kNN, HOST_SIZES>(p, hs, stream)
-                             : launch_dump<Short, gg::kNT, HOST_SIZES>(p, hs, stream);
+    return layout == gg::kNN ? launch_dump<Short, gg::kNN>(p, hs, stream)
+                             : launch_dump<Short, gg::kNT>(p, hs, stream);
   }
-  return layout == gg::kNN ? launch_dump<Wide, gg::kNN, HOST_SIZES>(p, hs, stream)
-                           : launch_dump<Wide, gg::kNT, HOST_SIZES>(p, hs, stream);
+  return layout == gg::kNN ? launch_dump<Wide, gg::kNN>(p, hs, stream)
+                           : launch_dump<Wide, gg::kNT>(p, hs, stream);
 }
 
 int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens, int64_t hidden_in,
@@ -184,17 +131,113 @@ int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens,
   return GG_OK;
 }
 
-// Upper bound of the tile count for any size vector (the device clips rows to `tokens`).
-int64_t tile_bound(int64_t num_groups, int64_t tokens, int64_t hidden_in, int64_t hidden_out,
-                   int trans_a, int bm, int bn) {
-  const int64_t tiles_n = (hidden_out + bn - 1) / bn;
-  if (trans_a) return num_groups * ((hidden_in + bm - 1) / bm) * tiles_n;
-  return (tokens / bm + num_groups) * tiles_n;
-}
+int gmm_impl(const gg_gmm_args& g) {
+  const int64_t num_groups = g.num_groups, tokens = g.tokens;
+  const int64_t hidden_in = g.hidden_in, hidden_out = g.hidden_out;
+  const int trans_a = g.trans_a != 0, trans_b = g.trans_b != 0;
+  const bool out_f32 = g.accumulate_f32 != 0;
+  int rc = check_common(g.batch_sizes, num_groups, tokens, hidden_in, hidden_out, trans_a, trans_b);
+  if (rc != GG_OK) return rc;
+  if (g.dtype != GG_DTYPE_BF16 && g.dtype != GG_DTYPE_F16)
+    return fail(GG_EINVAL, "dtype must be GG_DTYPE_BF16 or GG_DTYPE_F16");
+  if (out_f32 && !trans_a)
+    return fail(GG_EINVAL, "the fp32-accumulated output exists for the trans_a layout only");
+  if (out_f32 && (hidden_in >= (1 << 20) || hidden_out >= (1 << 20)))
+    return fail(GG_ELIMIT, "hidden sizes must be below 2^20 for the accumulating form");
+  if (num_groups == 0) return GG_OK;
+  // nothing to write
+  if (hidden_out == 0 || (trans_a ? hidden_in == 0 : tokens == 0)) return GG_OK;
+  if (g.c == nullptr) return fail(GG_EINVAL, "c is null");
+  if (tokens > 0 && (g.a == nullptr || g.b == nullptr)) return fail(GG_EINVAL, "a or b is null");
+  // rows are fetched and stored 16 bytes at a time
+  if ((reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b) | reinterpret_cast<uintptr_t>(g.c)) & 15)
+    return fail(GG_ELIMIT, "a, b and c must be 16-byte aligned");
 
-int gmm_impl(const void* a, const void* b, void* c, bool out_f32, const int64_t* batch_sizes,
-             int batch_sizes_on_device, int64_t num_groups, int64_t tokens, int64_t hidden_in,
-             int64_t hidden_out, int trans_a, int trans_b, void* stream_);
+  // Host-resident sizes are validated here; they travel in the kernel argument block.
+  if (!g.batch_sizes_on_device) {
+    int64_t row = 0;
+    for (int64_t e = 0; e < num_groups; ++e) {
+      if (g.batch_sizes[e] < 0) return fail(GG_EINVAL, "batch_sizes[%lld] is negative", (long long)e);
+      if (g.batch_sizes[e] > tokens - row)
+        return fail(GG_EINVAL, "batch_sizes sum past the %lld rows of a", (long long)tokens);
+      row += g.batch_sizes[e];
+    }
+  }
+
+  DeviceInfo info;
+  rc = device_info(&info);
+  if (rc != GG_OK) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(g.stream);
+  const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
+  const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
+  const int bm = short_shape ? Short::BM : Wide::BM, bn = short_shape ? Short::BN : Wide::BN;
+  const gg::VariantOps* variant = find_variant(g.dtype == GG_DTYPE_F16 ? gg::kF16 : gg::kBF16, layout,
+                                               short_shape ? Short::kId : Wide::kId,
+                                               out_f32 ? gg::kEpiAccF32 : gg::kEpiStore);
+  if (variant == nullptr) return fail(GG_EINVAL, "no kernel for this combination of arguments");
+
+  gg::GmmParams p{};
+  p.a = static_cast<const char*>(g.a);
+  p.b = static_cast<const char*>(g.b);
+  p.c = static_cast<char*>(g.c);
+  p.tokens = tokens;
+  p.hidden_in = (int32_t)hidden_in;
+  p.hidden_out = (int32_t)hidden_out;
+  p.group_m = band_height(num_groups, tokens, trans_a);
+  static_assert(GG_FLAG_WHOLE_TILES == gg::kFlagWholeTiles && GG_FLAG_ONE_CLASS == gg::kFlagOneClass &&
+                GG_FLAG_ROW_PIECES == gg::kFlagRowPieces, "the header's flags are the kernel's");
+  p.flags = g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ONE_CLASS | GG_FLAG_ROW_PIECES);
+  p.sched_out = nullptr;
+  if (g.workspace != nullptr) {
+    if (reinterpret_cast<uintptr_t>(g.workspace) & 255)
+      return fail(GG_ELIMIT, "the workspace must be 256-byte aligned");
+    const uint64_t slot_bytes = (uint64_t)bm * bn * 4;
+    if (g.workspace_bytes < gg::kWsCounterBytes + slot_bytes)
+      return fail(GG_ELIMIT, "the workspace holds %llu bytes, the smallest useful one %llu",
+                  (unsigned long long)g.workspace_bytes, (unsigned long long)(gg::kWsCounterBytes + slot_bytes));
+    const uint64_t slots = (g.workspace_bytes - gg::kWsCounterBytes) / slot_bytes;
+    p.workspace = static_cast<char*>(g.workspace);
+    // one arrival counter per tile of the last round: at most grid / 2 of them, 1024 fit
+    p.ws_slots = slots > 1024 ? 1024 : (int32_t)slots;
+  }
+
+  const int64_t tiles_n = (hidden_out + bn - 1) / bn;
+  const int64_t tiles_m_fixed = (hidden_in + bm - 1) / bm;   // weight-gradient layout
+  // At most GG_MAX_GROUPS_PER_LAUNCH groups per launch.  A launch sees all operands and the rows
+  // its groups start at: handed over by the host for host-resident sizes, summed up by the kernel
+  // itself from the sizes of the groups before it for device-resident ones.
+  int64_t row = 0;
+  for (int64_t first = 0; first < num_groups; first += GG_MAX_GROUPS_PER_LAUNCH) {
+    const int64_t count = num_groups - first < GG_MAX_GROUPS_PER_LAUNCH
+                              ? num_groups - first : GG_MAX_GROUPS_PER_LAUNCH;
+    gg::HostSizes hs;
+    p.first_group = (int32_t)first;
+    p.num_groups = (int32_t)count;
+    int64_t tiles;
+    if (g.batch_sizes_on_device) {
+      p.sizes_dev = g.batch_sizes;
+      p.row_base = 0;
+      // upper bound for any size vector (the device clips rows to `tokens`)
+      tiles = trans_a ? count * tiles_m_fixed * tiles_n : (tokens / bm + count) * tiles_n;
+    } else {
+      p.sizes_dev = nullptr;
+      p.row_base = row;
+      tiles = 0;
+      for (int64_t i = 0; i < count; ++i) {
+        const int64_t m = g.batch_sizes[first + i];
+        hs.v[i] = (int32_t)m;
+        row += m;
+        tiles += trans_a ? tiles_m_fixed * tiles_n : ((m + bm - 1) / bm) * tiles_n;
+      }
+    }
+    if (tiles >= (int64_t(1) << 31)) return fail(GG_ELIMIT, "too many output tiles for one launch");
+    if (tiles == 0) continue;
+    // the full grid also for few tiles: the last round's tiles may be cut into pieces for
+    // the workgroups that would otherwise idle
+    GG_HIP(variant->launch(p, hs, info.cus, stream));
+  }
+  return GG_OK;
+}
 
 }  // namespace
 
@@ -202,7 +245,12 @@ extern "C" {
 
 const char* gg_last_error(void) { return g_err; }
 
-int gg_version(void) { return 100; }
+int gg_version(void) { return 200; }
+
+int gg_init(void) {
+  DeviceInfo info;
+  return device_info(&info);
+}
 
 int gg_tile_shape(int64_t num_groups, int64_t tokens, int trans_a, int trans_b, int* bm, int* bn,
                   int* bk) {
@@ -210,123 +258,45 @@ int gg_tile_shape(int64_t num_groups, int64_t tokens, int trans_a, int trans_b, 
   const bool s = use_short_shape(num_groups, tokens, trans_a);
   if (bm) *bm = s ? Short::BM : Wide::BM;
   if (bn) *bn = s ? Short::BN : Wide::BN;
-  if (bk) *bk = BK;
+  if (bk) *bk = gg::BK;
   return GG_OK;
+}
+
+int gg_gmm(const gg_gmm_args* args) {
+  if (args == nullptr) return fail(GG_EINVAL, "args is null");
+  if (args->struct_bytes != sizeof(gg_gmm_args))
+    return fail(GG_EINVAL, "gg_gmm_args.struct_bytes is %u, this library expects %zu", args->struct_bytes,
+                sizeof(gg_gmm_args));
+  return gmm_impl(*args);
 }
 
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,
                 int batch_sizes_on_device, int64_t num_groups, int64_t tokens, int64_t hidden_in,
-                int64_t hidden_out, int trans_a, int trans_b, void* stream_) {
-  return gmm_impl(a, b, c, /*out_f32=*/false, batch_sizes, batch_sizes_on_device, num_groups, tokens,
-                  hidden_in, hidden_out, trans_a, trans_b, stream_);
+                int64_t hidden_out, int trans_a, int trans_b, void* stream) {
+  gg_gmm_args g{};
+  g.struct_bytes = sizeof(g);
+  g.dtype = GG_DTYPE_BF16;
+  g.a = a, g.b = b, g.c = c;
+  g.batch_sizes = batch_sizes, g.batch_sizes_on_device = batch_sizes_on_device;
+  g.num_groups = num_groups, g.tokens = tokens, g.hidden_in = hidden_in, g.hidden_out = hidden_out;
+  g.trans_a = trans_a, g.trans_b = trans_b;
+  g.stream = stream;
+  return gmm_impl(g);
 }
 
 int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* batch_sizes,
                         int batch_sizes_on_device, int64_t num_groups, int64_t tokens,
-                        int64_t hidden_in, int64_t hidden_out, void* stream_) {
-  if (hidden_in >= (1 << 20) || hidden_out >= (1 << 20))
-    return fail(GG_ELIMIT, "hidden sizes must be below 2^20 for the accumulating form");
-  return gmm_impl(a, b, c, /*out_f32=*/true, batch_sizes, batch_sizes_on_device, num_groups, tokens,
-                  hidden_in, hidden_out, /*trans_a=*/1, /*trans_b=*/0, stream_);
+                        int64_t hidden_in, int64_t hidden_out, void* stream) {
+  gg_gmm_args g{};
+  g.struct_bytes = sizeof(g);
+  g.dtype = GG_DTYPE_BF16;
+  g.a = a, g.b = b, g.c = c;
+  g.batch_sizes = batch_sizes, g.batch_sizes_on_device = batch_sizes_on_device;
+  g.num_groups = num_groups, g.tokens = tokens, g.hidden_in = hidden_in, g.hidden_out = hidden_out;
+  g.trans_a = 1, g.accumulate_f32 = 1;
+  g.stream = stream;
+  return gmm_impl(g);
 }
-
-}  // extern "C"
-
-namespace {
-
-int gmm_impl(const void* a, const void* b, void* c, bool out_f32, const int64_t* batch_sizes,
-             int batch_sizes_on_device, int64_t num_groups, int64_t tokens, int64_t hidden_in,
-             int64_t hidden_out, int trans_a, int trans_b, void* stream_) {
-  int rc = check_common(batch_sizes, num_groups, tokens, hidden_in, hidden_out, trans_a, trans_b);
-  if (rc != GG_OK) return rc;
-  if (num_groups == 0) return GG_OK;
-  // nothing to write
-  if (hidden_out == 0 || (trans_a ? hidden_in == 0 : tokens == 0)) return GG_OK;
-  if (c == nullptr) return fail(GG_EINVAL, "c is null");
-  if (tokens > 0 && (a == nullptr || b == nullptr)) return fail(GG_EINVAL, "a or b is null");
-  // rows are fetched and stored 16 bytes at a time
-  if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c)) & 15)
-    return fail(GG_ELIMIT, "a, b and c must be 16-byte aligned");
-  if (batch_sizes_on_device && num_groups > GG_MAX_GROUPS_PER_LAUNCH)
-    return fail(GG_ELIMIT, "at most %d groups are supported when batch_sizes is on the device, got %lld",
-                GG_MAX_GROUPS_PER_LAUNCH, (long long)num_groups);
-
-  DeviceInfo info;
-  rc = device_info(&info);
-  if (rc != GG_OK) return rc;
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
-
-  gg::GmmParams p{};
-  p.tokens = tokens;
-  p.hidden_in = (int32_t)hidden_in;
-  p.hidden_out = (int32_t)hidden_out;
-  p.group_m = band_height(num_groups, tokens, trans_a);
-  p.tail_split = tail_split();
-  p.sched_out = nullptr;
-
-  const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
-  const int bm = short_shape ? Short::BM : Wide::BM, bn = short_shape ? Short::BN : Wide::BN;
-  if (batch_sizes_on_device) {
-    if (tile_bound(num_groups, tokens, hidden_in, hidden_out, trans_a, bm, bn) >= (int64_t(1) << 31))
-      return fail(GG_ELIMIT, "too many output tiles for one launch");
-    p.a = static_cast<const char*>(a);
-    p.b = static_cast<const char*>(b);
-    p.c = static_cast<char*>(c);
-    p.sizes_dev = batch_sizes;
-    p.num_groups = (int32_t)num_groups;
-    return dispatch<false>(short_shape, layout, out_f32, p, nullptr, info.cus, stream);
-  }
-
-  // Host-resident sizes: validated here, passed in the kernel argument block, at most
-  // GG_MAX_GROUPS_PER_LAUNCH groups per launch.
-  int64_t row = 0;
-  for (int64_t e = 0; e < num_groups; ++e) {
-    if (batch_sizes[e] < 0) return fail(GG_EINVAL, "batch_sizes[%lld] is negative", (long long)e);
-    row += batch_sizes[e];
-    if (row > tokens)
-      return fail(GG_EINVAL, "batch_sizes sum past the %lld rows of a", (long long)tokens);
-  }
-  row = 0;
-  for (int64_t first = 0; first < num_groups; first += GG_MAX_GROUPS_PER_LAUNCH) {
-    const int64_t count = num_groups - first < GG_MAX_GROUPS_PER_LAUNCH
-                              ? num_groups - first : GG_MAX_GROUPS_PER_LAUNCH;
-    gg::HostSizes hs;
-    int64_t rows_here = 0, tiles = 0;
-    const int64_t tiles_n = (hidden_out + bn - 1) / bn;
-    for (int64_t i = 0; i < count; ++i) {
-      hs.v[i] = (int32_t)batch_sizes[first + i];
-      rows_here += batch_sizes[first + i];
-      tiles += trans_a ? ((hidden_in + bm - 1) / bm) * tiles_n
-                       : ((batch_sizes[first + i] + bm - 1) / bm) * tiles_n;
-    }
-    if (tiles >= (int64_t(1) << 31)) return fail(GG_ELIMIT, "too many output tiles for one launch");
-    // this launch sees its own groups as groups 0..count-1 of operands that start at `row`
-    p.tokens = rows_here;
-    p.num_groups = (int32_t)count;
-    p.sizes_dev = nullptr;
-    p.a = static_cast<const char*>(a) + row * hidden_in * 2;
-    if (trans_a) {
-      p.b = static_cast<const char*>(b) + row * hidden_out * 2;
-      p.c = static_cast<char*>(c) + first * hidden_in * hidden_out * (out_f32 ? 4 : 2);
-    } else {
-      p.b = static_cast<const char*>(b) + first * hidden_in * hidden_out * 2;
-      p.c = static_cast<char*>(c) + row * hidden_out * 2;
-    }
-    if (tiles > 0) {
-      // the full grid also for few tiles: the last round's tiles may be cut into pieces for
-      // the workgroups that would otherwise idle
-      rc = dispatch<true>(short_shape, layout, out_f32, p, &hs, info.cus, stream);
-      if (rc != GG_OK) return rc;
-    }
-    row += rows_here;
-  }
-  return GG_OK;
-}
-
-}  // namespace
-
-extern "C" {
 
 int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int64_t num_groups,
                       int64_t tokens, int64_t hidden_in, int64_t hidden_out, int trans_a,
@@ -346,22 +316,21 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   p.hidden_in = (int32_t)hidden_in;
   p.hidden_out = (int32_t)hidden_out;
   p.group_m = band_height(num_groups, tokens, trans_a);
-  p.tail_split = tail_split();
   p.num_groups = (int32_t)num_groups;
   p.sched_out = table_out;
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
   const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
+  gg::HostSizes hs;
   if (batch_sizes_on_device) {
     p.sizes_dev = batch_sizes;
-    return dispatch_dump<false>(short_shape, layout, p, nullptr, stream);
+  } else {
+    // the table shows what the kernel would do with these sizes: clamped like device-resident ones
+    for (int64_t i = 0; i < num_groups; ++i) {
+      const int64_t v = batch_sizes[i];
+      hs.v[i] = (int32_t)(v < 0 ? 0 : (v > tokens ? tokens : v));
+    }
   }
-  gg::HostSizes hs;
-  for (int64_t i = 0; i < num_groups; ++i) {
-    if (batch_sizes[i] < 0 || batch_sizes[i] >= (int64_t(1) << 31))
-      return fail(GG_EINVAL, "batch_sizes[%lld] out of range", (long long)i);
-    hs.v[i] = (int32_t)batch_sizes[i];
-  }
-  return dispatch_dump<true>(short_shape, layout, p, &hs, stream);
+  return dispatch_dump(short_shape, layout, p, hs, stream);
 }
 
 }  // extern "C"

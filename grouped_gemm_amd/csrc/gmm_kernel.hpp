@@ -27,12 +27,15 @@
 namespace gg {
 
 constexpr int kMaxGroups = 512;
-constexpr int kSchedCols = 12;
+constexpr int kSchedCols = 14;
 
 enum : int { kNN = 0, kNT = 1, kTN = 2 };
+enum : int { kBF16 = 0, kF16 = 1 };   // element type of the operands, two bytes either way
 
 using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
 using bf16x4 = __attribute__((ext_vector_type(4))) __bf16;
+using f16x8 = __attribute__((ext_vector_type(8))) _Float16;
+using f16x4 = __attribute__((ext_vector_type(4))) _Float16;
 using f32x16 = __attribute__((ext_vector_type(16))) float;
 using f32x4 = __attribute__((ext_vector_type(4))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) uint32_t;
@@ -44,30 +47,73 @@ struct GmmParams {
   const char* a;
   const char* b;
   char* c;
-  const int64_t* sizes_dev;  // device-resident batch_sizes, or nullptr
+  const int64_t* sizes_dev;  // device-resident batch_sizes of ALL groups, or nullptr (then HostSizes)
   int64_t* sched_out;        // only read by the schedule dump kernel
+  char* workspace;           // counters + fp32 partial tiles of depth pieces, or nullptr
   int64_t tokens;            // rows of a
-  int32_t num_groups;
+  int64_t row_base;          // host-resident sizes: rows taken by the groups before first_group
+  int32_t first_group;       // this launch schedules groups first_group .. first_group + num_groups - 1
+  int32_t num_groups;        // at most kMaxGroups
   int32_t hidden_in;
   int32_t hidden_out;
-  int32_t group_m;  // tile rows per band of the in-group tile order
-  int32_t tail_split;  // 1: the tiles of the last, partly filled round may be cut into row pieces
+  int32_t group_m;     // tile rows per band of the in-group tile order
+  int32_t flags;       // kFlag* bits
+  int32_t ws_slots;    // partial-tile slots the workspace holds (0: no depth pieces)
 };
 
+enum : int {   // debugging switches, for comparing the ways a call can be scheduled
+  kFlagWholeTiles = 1,    // never cut the tiles of the last round into pieces
+  kFlagOneClass = 2,      // hand out runt rows in place, not after all other tiles
+  kFlagRowPieces = 4,     // ignore the workspace: cut along the rows only
+};
+
+// Workspace layout: kWsCounterBytes of int32 arrival counters (one per tile of the last round; all
+// zero before a launch and all zero again after it), then ws_slots partial tiles of BM x BN floats.
+constexpr int kWsCounterBytes = 4096;
+// Depth pieces per tile: 2 or 4.  A piece's fix-up (a partial tile written, the last piece reading
+// them all back) costs about as much as 20 depth slices, so only deep tiles are cut.
+constexpr int kMaxDepthPieces = 4;
+constexpr int kMinSlicesPerPiece = 48;
+
 // The last round of a persistent grid is filled only partly: `tiles % grid` workgroups have a
-// tile, the others idle.  When that rest is at most half (a quarter) of the grid, each of its
-// tiles is cut along its rows into 2 (4) pieces that go to different workgroups; a piece issues
-// MFMAs only for its own 32-row blocks, so the round ends sooner.  A launch with fewer tiles
-// than workgroups is all "last round".
+// tile, the others idle.  When that rest is at most half of the grid, each of its tiles is cut
+// into pieces that go to different workgroups.  With a workspace (and a deep product) the cut
+// runs along the depth:
+// every piece accumulates its share of the depth slices into an fp32 partial tile in the
+// workspace, and the piece that arrives last adds the partial tiles up in piece order (so the sum
+// does not depend on which piece that is) and stores the result.  Without a workspace the cut
+// runs along the rows (2 or 4 pieces of whole 32-row blocks; not in the weight-gradient layout).
+// A launch with fewer tiles than workgroups is all "last round".
 struct TailPlan {
   int main_tiles;   // tiles before the last round, handed out whole
-  int pieces;       // pieces per tile of the last round: 1, 2 or 4
+  int pieces;       // pieces per tile of the last round
   int total;        // indices to hand out: main_tiles + rest * pieces
+  bool by_depth;
 };
-__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, bool enabled) {
+template <int LAYOUT>
+__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmParams& p, int bk) {
   TailPlan t;
   const int rest = tiles % grid;
-  t.pieces = !enabled || rest == 0 ? 1 : (4 * rest <= grid ? 4 : (2 * rest <= grid ? 2 : 1));
+  t.pieces = 1;
+  t.by_depth = false;
+  if (rest > 0 && 2 * rest <= grid && !(p.flags & kFlagWholeTiles)) {
+    int cand = grid / rest;
+    cand = cand > kMaxDepthPieces ? kMaxDepthPieces : cand;
+    if (p.ws_slots > 0 && !(p.flags & kFlagRowPieces)) {
+      if (rest * cand > p.ws_slots) cand = p.ws_slots / rest;
+      cand = cand >= 4 ? 4 : cand;
+      if (LAYOUT != kTN) {   // the depth is the same for every tile: keep the pieces worth their fix-up
+        const int nk = (p.hidden_in + bk - 1) / bk;
+        if (cand > nk / kMinSlicesPerPiece) cand = nk / kMinSlicesPerPiece;
+      }
+      cand &= ~1;   // 2 or 4 (3 becomes 2): the fix-up sums two pieces per step
+      if (cand >= 2) {
+        t.pieces = cand;
+        t.by_depth = true;
+      }
+    }
+    if (!t.by_depth && LAYOUT != kTN) t.pieces = 4 * rest <= grid ? 4 : 2;
+  }
   t.main_tiles = t.pieces > 1 ? tiles - rest : tiles;
   t.total = t.main_tiles + (tiles - t.main_tiles) * t.pieces;
   return t;
@@ -77,13 +123,18 @@ __device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, bool enabled)
 struct HostSizes {
   int32_t v[kMaxGroups];
 };
-struct NoSizes {};
 
-// What every workgroup keeps in LDS about the groups.
+// What every workgroup keeps in LDS about the groups.  Tiles come in two classes: first all
+// tiles except each group's last, much shorter tile row ("runt" row: at most half the 32-row
+// blocks of the group's other tile rows), then the runt rows.  Tiles of one class take about the
+// same time, so workgroups that walk the classes in this order stay in step, and the cheap tiles
+// fill the end of the launch.
 struct Sched {
   int32_t row_start[kMaxGroups + 1];   // exclusive prefix sum of rows, clipped to tokens
   int32_t rows[kMaxGroups];            // rows of `a` the group uses
-  int32_t tile_start[kMaxGroups + 1];  // exclusive prefix sum of tiles
+  int32_t tile_start[kMaxGroups + 1];  // exclusive prefix sum of the first class's tiles
+  int32_t runt_start[kMaxGroups + 1];  // exclusive prefix sum of the runt rows' tiles
+  int32_t arrived;                     // broadcast slot for the arrival count of a depth piece
 };
 
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor size used here
@@ -129,7 +180,7 @@ __device__ __forceinline__ void load_to_lds_16(const rsrc_words& rsrc, uint32_t 
       "buffer_load_dwordx4 %0, %1, 0 offen lds"
       :
       : "v"(voffset), "s"(rsrc), "s"(lds_addr)
-      : "memory");
+      : "memory", "m0");
 }
 
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
@@ -148,24 +199,87 @@ __device__ __forceinline__ void block_barrier() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// One 32x32x16 matrix instruction on fragments of 8 two-byte elements per lane (carried as
+// bf16x8 whatever the element type; the type only selects the instruction).
+template <int DT>
+__device__ __forceinline__ f32x16 mfma_32x32x16(bf16x8 x, bf16x8 y, f32x16 acc) {
+  if constexpr (DT == kBF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, acc, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, x),
+                                                  __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
+  }
+}
+
+// Four fp32 values rounded (to nearest even) to the element type, as 8 bytes.
+template <int DT>
+__device__ __forceinline__ u32x2 round4(float v0, float v1, float v2, float v3) {
+  if constexpr (DT == kBF16) {
+    bf16x4 o = {(__bf16)v0, (__bf16)v1, (__bf16)v2, (__bf16)v3};
+    return __builtin_bit_cast(u32x2, o);
+  } else {
+    f16x4 o = {(_Float16)v0, (_Float16)v1, (_Float16)v2, (_Float16)v3};
+    return __builtin_bit_cast(u32x2, o);
+  }
+}
+
 // ---------------------------------------------------------------------- schedule
 
+// How a group's output is cut into tiles.
+struct GroupTiles {
+  int tiles_m, tiles_n;
+  int height;       // rows per tile row (the last tile row takes what is left)
+  int main_rows;    // tile rows of the first class
+  int runt;         // 1: the last tile row is a runt row (second class)
+};
+
+// The rows of a group are split evenly over its tile rows, in whole 32-row blocks: 300 rows make
+// two tile rows of 160 (5 blocks each), not one of 256 and one of 44.  Tile rows of a group then
+// take the same time, and blocks without rows cost nothing.  What is left for the last tile row
+// of a tall group can still be much less than the others' (4122 rows: 16 tile rows of 256 and one
+// of 26): such a row goes to the second class.
 template <int LAYOUT, int BM, int BN>
-__device__ __forceinline__ int tiles_of_group(int rows, int hidden_in, int hidden_out) {
-  const int tiles_n = (hidden_out + BN - 1) / BN;
-  if (LAYOUT == kTN) return ((hidden_in + BM - 1) / BM) * tiles_n;
-  return ((rows + BM - 1) / BM) * tiles_n;
+__device__ __forceinline__ GroupTiles group_tiles(int rows, int hidden_in, int hidden_out, int flags) {
+  GroupTiles g;
+  g.tiles_n = (hidden_out + BN - 1) / BN;
+  g.runt = 0;
+  if (LAYOUT == kTN) {
+    g.tiles_m = (hidden_in + BM - 1) / BM;
+    g.height = BM;
+  } else {
+    g.tiles_m = (rows + BM - 1) / BM;
+    g.height = BM;
+    if (g.tiles_m > 0) {
+      g.height = ((rows + g.tiles_m - 1) / g.tiles_m + 31) / 32 * 32;
+      const int last_blocks = (rows - (g.tiles_m - 1) * g.height + 31) / 32;
+      g.runt = g.tiles_m >= 2 && 2 * last_blocks <= g.height / 32 && !(flags & kFlagOneClass) ? 1 : 0;
+    }
+  }
+  g.main_rows = g.tiles_m - g.runt;
+  return g;
 }
 
 // Run by the first wave of a workgroup.  Each lane owns up to 8 consecutive groups; one
-// wave-wide scan of int64 row counts and one of int32 tile counts.
-template <int LAYOUT, int BM, int BN, bool HOST_SIZES, typename SizesArg>
-__device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, const SizesArg& hs) {
+// wave-wide scan of int64 row counts and one of the two int32 tile counts.  Every size is
+// clamped to [0, tokens] before it enters a sum, so no size vector can make a sum overflow or a
+// group start before row 0 or end past row `tokens`.
+template <int LAYOUT, int BM, int BN>
+__device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, const HostSizes& hs) {
   const int lane = threadIdx.x;
   if (lane >= 64) return;
   const int E = p.num_groups;
   const int per = (E + 63) >> 6;
   const int e0 = lane * per;
+  auto clamp = [&](int64_t v) { return v < 0 ? (int64_t)0 : (v > p.tokens ? p.tokens : v); };
+  // rows taken by the groups before this launch's first one
+  int64_t base = p.row_base;
+  if (p.sizes_dev != nullptr && p.first_group > 0) {
+    int64_t part = 0;
+    for (int i = lane; i < p.first_group; i += 64) part += clamp(p.sizes_dev[i]);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) part += __shfl_xor(part, d);
+    base = part;
+  }
   int64_t sz[8];
   int64_t sum = 0;
 #pragma unroll
@@ -173,12 +287,8 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
     const int e = e0 + i;
     int64_t v = 0;
     if (i < per && e < E) {
-      if constexpr (HOST_SIZES) {
-        v = hs.v[e];
-      } else {
-        v = p.sizes_dev[e];
-      }
-      v = v < 0 ? 0 : v;
+      v = p.sizes_dev != nullptr ? p.sizes_dev[p.first_group + e] : (int64_t)hs.v[e];
+      v = clamp(v);
     }
     sz[i] = v;
     sum += v;
@@ -189,9 +299,9 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
     const int64_t o = __shfl_up(incl, d);
     if (lane >= d) incl += o;
   }
-  int64_t run = incl - sum;
+  int64_t run = base + incl - sum;
   int rows[8];
-  int tsum = 0;
+  int tsum = 0, rsum = 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int e = e0 + i;
@@ -202,28 +312,38 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
     if (i < per && e < E) {
       s->row_start[e] = (int)start;
       s->rows[e] = r;
-      tsum += tiles_of_group<LAYOUT, BM, BN>(r, p.hidden_in, p.hidden_out);
+      const GroupTiles g = group_tiles<LAYOUT, BM, BN>(r, p.hidden_in, p.hidden_out, p.flags);
+      tsum += g.main_rows * g.tiles_n;
+      rsum += g.runt * g.tiles_n;
     }
     run += sz[i];
   }
-  int tincl = tsum;
+  int tincl = tsum, rincl = rsum;
 #pragma unroll
   for (int d = 1; d < 64; d <<= 1) {
     const int o = __shfl_up(tincl, d);
-    if (lane >= d) tincl += o;
+    const int o2 = __shfl_up(rincl, d);
+    if (lane >= d) {
+      tincl += o;
+      rincl += o2;
+    }
   }
-  int trun = tincl - tsum;
+  int trun = tincl - tsum, rrun = rincl - rsum;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int e = e0 + i;
     if (i < per && e < E) {
       s->tile_start[e] = trun;
-      trun += tiles_of_group<LAYOUT, BM, BN>(rows[i], p.hidden_in, p.hidden_out);
+      s->runt_start[e] = rrun;
+      const GroupTiles g = group_tiles<LAYOUT, BM, BN>(rows[i], p.hidden_in, p.hidden_out, p.flags);
+      trun += g.main_rows * g.tiles_n;
+      rrun += g.runt * g.tiles_n;
     }
   }
   if (lane == 63) {
     s->row_start[E] = (int)(run < p.tokens ? run : p.tokens);
     s->tile_start[E] = tincl;
+    s->runt_start[E] = rincl;
   }
 }
 
@@ -235,7 +355,8 @@ struct GroupGeom {
   int32_t m, n, k;
 };
 
-// `start` and `rows` are the group's entries of Sched::row_start and Sched::rows.
+// `e` is the group's index among all groups of the call; `start` and `rows` are the group's
+// entries of Sched::row_start and Sched::rows.
 template <int LAYOUT>
 __device__ __forceinline__ GroupGeom group_geometry(const GmmParams& p, int e, int64_t start,
                                                     int rows) {
@@ -273,14 +394,14 @@ __device__ __forceinline__ void tile_coords(int u, int tiles_m, int tiles_n, int
   *tn = r / gsz;
 }
 
-template <int LAYOUT, int BM, int BN, bool HOST_SIZES>
-__global__ __launch_bounds__(64) void schedule_dump_kernel(
-    GmmParams p, std::conditional_t<HOST_SIZES, HostSizes, NoSizes> hs) {
+template <int LAYOUT, int BM, int BN>
+__global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSizes hs) {
   __shared__ Sched s;
-  build_schedule<LAYOUT, BM, BN, HOST_SIZES>(&s, p, hs);
+  build_schedule<LAYOUT, BM, BN>(&s, p, hs);
   __syncthreads();
   for (int e = threadIdx.x; e < p.num_groups; e += 64) {
-    const GroupGeom g = group_geometry<LAYOUT>(p, e, s.row_start[e], s.rows[e]);
+    const GroupGeom g = group_geometry<LAYOUT>(p, p.first_group + e, s.row_start[e], s.rows[e]);
+    const GroupTiles gt = group_tiles<LAYOUT, BM, BN>(s.rows[e], p.hidden_in, p.hidden_out, p.flags);
     int64_t* row = p.sched_out + (int64_t)e * kSchedCols;
     row[0] = g.m;
     row[1] = g.n;
@@ -292,8 +413,10 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(
     row[7] = g.b_off;
     row[8] = g.c_off;
     row[9] = s.tile_start[e];
-    row[10] = s.tile_start[e + 1] - s.tile_start[e];
+    row[10] = gt.tiles_m * gt.tiles_n;
     row[11] = s.rows[e];
+    row[12] = s.tile_start[p.num_groups] + s.runt_start[e];
+    row[13] = gt.runt * gt.tiles_n;
   }
 }
 
@@ -503,24 +626,38 @@ struct GmmConfig {
   static_assert(BK % 16 == 0 && STAGES >= 2, "");
 };
 
-// One output tile as the scheduler hands it out.
+// One output tile (or one piece of a tile of the last round) as the scheduler hands it out.
 struct TileInfo {
   GroupGeom g;
   int m0, n0;       // first row and column of the tile inside its group's output
   int rows_valid;   // rows of the tile that exist (0: no tile)
   int blocks;       // 32-row blocks the tile's rows take (MFMAs are issued for these only)
   int depth;        // depth to fetch (0: nothing to fetch, the tile multiplies zeros)
+  int k0;           // first depth slice (not 0 only for a depth piece)
   int nk;           // depth slices, at least 1 so that an empty group still stores zeros
+  int pieces;       // depth pieces this tile is cut into (1: whole depth, store directly)
+  int piece;        // which of them this is
+  int rank;         // index of the tile among the tiles of the last round
   bool valid;
 };
 
-// Tile index -> group and position.  `e` is the caller's cursor into the groups; tile
-// indices only grow, so it only moves forward.  Indices past plan.main_tiles name pieces of the
-// last round's tiles: piece (t - main) % pieces of tile main + (t - main) / pieces.
+// Where a tile cursor stands: group and class.  Tile indices only grow, so inside a class the
+// group only moves forward; it starts over once, when the indices pass into the runt class.
+struct TileCursor {
+  int e = 0;
+  int cls = 0;
+};
+
+// Tile index -> group and position.  Indices past plan.main_tiles name pieces of the last
+// round's tiles: piece (t - main) % pieces of tile main + (t - main) / pieces.
 template <int LAYOUT, int BM, int BN, int BK>
 __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParams& p, int t,
-                                              const TailPlan& plan, int& e) {
+                                              const TailPlan& plan, TileCursor& cur) {
   TileInfo ti;
+  ti.k0 = 0;
+  ti.pieces = 1;
+  ti.piece = 0;
+  ti.rank = 0;
   if (t >= plan.total) {
     ti.g = GroupGeom{0, 0, 0, 0, 0, 0};
     ti.m0 = ti.n0 = ti.rows_valid = ti.depth = 0;
@@ -533,28 +670,54 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   if (t >= plan.main_tiles) {
     const int r = t - plan.main_tiles;
     piece = r % plan.pieces;
-    t = plan.main_tiles + r / plan.pieces;
+    ti.rank = r / plan.pieces;
+    t = plan.main_tiles + ti.rank;
   }
-  while (t >= uniform(sched->tile_start[e + 1])) ++e;
+  const int first_class = uniform(sched->tile_start[p.num_groups]);
+  int u;
+  if (t < first_class) {
+    while (t >= uniform(sched->tile_start[cur.e + 1])) ++cur.e;
+    u = t - uniform(sched->tile_start[cur.e]);
+  } else {
+    if (cur.cls == 0) {
+      cur.cls = 1;
+      cur.e = 0;
+    }
+    t -= first_class;
+    while (t >= uniform(sched->runt_start[cur.e + 1])) ++cur.e;
+    u = t - uniform(sched->runt_start[cur.e]);
+  }
+  const int e = cur.e;
   // read through the first lane: everything derived from these stays in scalar registers
-  ti.g = group_geometry<LAYOUT>(p, e, uniform(sched->row_start[e]), uniform(sched->rows[e]));
-  const int u = t - uniform(sched->tile_start[e]);
-  const int tiles_n = (ti.g.n + BN - 1) / BN;
-  const int tiles_m = (ti.g.m + BM - 1) / BM;
+  const int rows = uniform(sched->rows[e]);
+  ti.g = group_geometry<LAYOUT>(p, p.first_group + e, uniform(sched->row_start[e]), rows);
+  const GroupTiles gt = group_tiles<LAYOUT, BM, BN>(rows, p.hidden_in, p.hidden_out, p.flags);
   int tm, tn;
-  tile_coords(u, tiles_m, tiles_n, p.group_m, &tm, &tn);
-  // The rows of a group are split evenly over its tiles, in whole 32-row blocks: 300 rows
-  // make two tiles of 160 (5 blocks each), not one of 256 and one of 44.  Tiles of a group then
-  // take the same time, and blocks without rows cost nothing.
-  int height = BM;
-  if (LAYOUT != kTN && tiles_m > 0) height = ((ti.g.m + tiles_m - 1) / tiles_m + 31) / 32 * 32;
-  ti.m0 = uniform(tm) * height;
+  if (cur.cls == 0) {
+    tile_coords(u, gt.main_rows, gt.tiles_n, p.group_m, &tm, &tn);
+  } else {
+    tm = gt.tiles_m - 1;
+    tn = u;
+  }
+  ti.m0 = uniform(tm) * gt.height;
   ti.n0 = uniform(tn) * BN;
-  ti.rows_valid = min(height, ti.g.m - ti.m0);
+  ti.rows_valid = min(gt.height, ti.g.m - ti.m0);
   ti.depth = ti.g.k;
   const int nk = (ti.g.k + BK - 1) / BK;
   ti.nk = nk < 1 ? 1 : nk;
-  if (piece >= 0) {
+  if (piece >= 0 && plan.by_depth) {
+    // this piece's share of the depth slices; a piece without slices contributes zeros
+    const int first = piece * ti.nk / plan.pieces, last = (piece + 1) * ti.nk / plan.pieces;
+    ti.pieces = plan.pieces;
+    ti.piece = piece;
+    ti.k0 = first;
+    ti.nk = last - first;
+    if (ti.nk <= 0) {
+      ti.k0 = 0;
+      ti.nk = 1;
+      ti.depth = 0;
+    }
+  } else if (piece >= 0) {
     // this piece's share of the tile's 32-row blocks; a piece past the rows is an empty tile
     const int all = (ti.rows_valid + 31) / 32;
     const int per = (all + plan.pieces - 1) / plan.pieces;
@@ -574,10 +737,10 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
 
 // ACC_F32: c holds fp32 and the product is added to it (gradient accumulation); otherwise c
 // holds bf16 and is overwritten.
-template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N, bool HOST_SIZES,
+// DT: element type of a and b (and of c unless ACC_F32).
+template <int DT, int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N,
           bool ACC_F32 = false>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
-    GmmParams p, std::conditional_t<HOST_SIZES, HostSizes, NoSizes> hs) {
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p, HostSizes hs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
   constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB, KS = BK / 16;
@@ -593,7 +756,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   Sched* sched = reinterpret_cast<Sched*>(smem + Cfg::SCHED_OFFSET);
-  build_schedule<LAYOUT, BM, BN, HOST_SIZES>(sched, p, hs);
+  build_schedule<LAYOUT, BM, BN>(sched, p, hs);
   __syncthreads();
 
   const int lane = threadIdx.x & 63;
@@ -605,9 +768,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   afrag.setup(wm * 32);   // wave row wm owns row blocks wm, wm + WAVES_M, ...
   bfrag.setup(wn * Cfg::WTN);
 
-  // (the weight-gradient layout has no ragged rows and no tile body for part of a tile)
-  const TailPlan plan = plan_tail(uniform(sched->tile_start[p.num_groups]), (int)gridDim.x,
-                                  LAYOUT != kTN && p.tail_split != 0);
+  const TailPlan plan = plan_tail<LAYOUT>(
+      uniform(sched->tile_start[p.num_groups]) + uniform(sched->runt_start[p.num_groups]),
+      (int)gridDim.x, p, BK);
   const int total_tiles = plan.total;
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
@@ -622,10 +785,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   // slices of a tile are already in flight while the previous tile is being stored.
   ALoad aload;
   BLoad bload;
-  int fetch_t = vid, fetch_e = 0, fetch_kt = 0;
+  int fetch_t = vid, fetch_kt = 0;
+  TileCursor fetch_cur;
   TileInfo fti;
   auto fetch_setup = [&]() {
-    fti = find_tile<LAYOUT, BM, BN, BK>(sched, p, fetch_t, plan, fetch_e);
+    fti = find_tile<LAYOUT, BM, BN, BK>(sched, p, fetch_t, plan, fetch_cur);
     const int depth = fti.depth;
     if constexpr (Cfg::A_DEPTH_MAJOR) {
       aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * 2, fti.g.k, fti.rows_valid, depth);
@@ -644,8 +808,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   typename ALoad::Slice a_slice;
   typename BLoad::Slice b_slice;
   auto fetch_begin = [&]() {   // descriptors of the cursor's slice
-    a_slice = aload.slice(fetch_kt);
-    b_slice = bload.slice(fetch_kt);
+    a_slice = aload.slice(fti.k0 + fetch_kt);
+    b_slice = bload.slice(fti.k0 + fetch_kt);
   };
   // Load J of the cursor's slice (A's loads first, then B's) into buffer `buf`.
   auto fetch_load = [&](auto j_tag, int buf) {
@@ -697,8 +861,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   fetch_begin();
   static_for<3 * QUARTER_LOADS>([&](auto j) { fetch_load(j, 1); });
 
-  int tile_t = vid, tile_e = 0;
-  TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_e);
+  int tile_t = vid;
+  TileCursor tile_cur;
+  TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_cur);
   wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
@@ -707,6 +872,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
   });
 
   int x = 0;   // buffer of the slice being multiplied
+
+  // Partial tile of depth piece `piece` of the tile `ti` names, as this thread sees it: a lane's
+  // 16-byte group (i, j, q) sits at ((i * NB + j) * 4 + q) * NT + thread, so one instruction of a
+  // wave moves 1 KiB of consecutive bytes.
+  auto partial_slot = [&](int piece) {
+    return reinterpret_cast<float*>(p.workspace + kWsCounterBytes) +
+           (int64_t)(ti.rank * ti.pieces + piece) * (BM * BN) + threadIdx.x * 4;
+  };
+  bool fix_pending = false;   // this workgroup's depth piece was the last of its tile to arrive
 
   // One tile, for a wave that has ML row blocks with rows in them (the tile's row blocks go to
   // the wave rows alternately).  One copy of this body exists per value of ML; a tile picks
@@ -748,7 +922,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
         constexpr int j = m / ML, i = (j % 2 == 0) ? m % ML : ML - 1 - m % ML;
         // operands swapped: the result block is held transposed, so a lane owns four
         // consecutive columns of one output row
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+        acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
         constexpr int u0 = READS * m / SLOTS, u1 = READS * (m + 1) / SLOTS;
         static_for<u1 - u0>([&](auto d) {
           constexpr int u = u0 + decltype(d)::value;
@@ -780,6 +954,28 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
       x = y;
     }
 
+    // A depth piece of a tile of the last round: park the partial tile in the workspace and
+    // count the arrival.  The piece that arrives last adds the partial tiles up and stores the
+    // sum, after the tile loop (fix_up below), where no accumulator is live any more.
+    if (ti.pieces > 1) {
+      float* mine = partial_slot(ti.piece);
+#pragma unroll
+      for (int i = 0; i < ML; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            f32x4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            *reinterpret_cast<f32x4*>(mine + ((i * NB + j) * 4 + q) * (NT * 4)) = v;
+          }
+      __threadfence();   // the partial tile is visible device-wide before the arrival is counted
+      block_barrier();
+      if (threadIdx.x == 0) sched->arrived = atomicAdd(reinterpret_cast<int*>(p.workspace) + ti.rank, 1);
+      block_barrier();
+      fix_pending = uniform(sched->arrived) == ti.pieces - 1;
+      return;
+    }
+
     // Epilogue.  A lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3.
     // The accumulators stay in the accumulation registers; each value is moved out right
     // where it is converted, so the epilogue needs only a few vector registers.
@@ -789,14 +985,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
       const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * (uint32_t)CE : 0u;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
       auto take4 = [&](int i, int j, int q) {
-        bf16x4 o;
+        float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v;
-          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
-          o[r] = (__bf16)v;
-        }
-        return __builtin_bit_cast(u32x2, o);
+        for (int r = 0; r < 4; ++r)
+          asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[r]) : "a"(acc[i][j][4 * q + r]));
+        return round4<DT>(v[0], v[1], v[2], v[3]);
       };
       if constexpr (ACC_F32) {
         // c += product in fp32.  The 4 consecutive columns a lane holds are 16 bytes of c:
@@ -902,9 +1095,63 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(
     }
     tile_t += G;
     if (tile_t >= total_tiles) break;
-    ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_e);
+    ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_cur);
   }
   wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
+
+  // Fix-up of a tile that was cut along the depth.  Pieces exist in the last round only, so a
+  // piece is its workgroup's last tile and `ti` still names it.  The partial tiles are added up
+  // in piece order, two per step (their count is even), whichever piece does the adding, so the
+  // result does not depend on timing.  One block row of 32 rows at a time: NB * 4 groups of 16
+  // bytes per lane and piece.
+  if (fix_pending) {
+    __threadfence();   // the other pieces' partial tiles are visible to this workgroup
+    if (threadIdx.x == 0) reinterpret_cast<int*>(p.workspace)[ti.rank] = 0;   // leave the counters as they were found
+    constexpr int CE = ACC_F32 ? 4 : 2;   // bytes per element of c
+    const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * CE;
+    const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * (uint32_t)CE : 0u;
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
+    const int live = LAYOUT == kTN ? MB : (ti.blocks - wm + WAVES_M - 1) / WAVES_M;
+    for (int i = 0; i < live; ++i) {
+      f32x4 sum[NB][4];
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sum[j][q] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      for (int piece = 0; piece < ti.pieces; piece += 2) {
+        const float* from0 = partial_slot(piece) + (i * NB * 4) * (NT * 4);
+        const float* from1 = partial_slot(piece + 1) + (i * NB * 4) * (NT * 4);
+        f32x4 v0[NB][4], v1[NB][4];
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            v0[j][q] = *reinterpret_cast<const f32x4*>(from0 + (j * 4 + q) * (NT * 4));
+            v1[j][q] = *reinterpret_cast<const f32x4*>(from1 + (j * 4 + q) * (NT * 4));
+          }
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) sum[j][q] = (sum[j][q] + v0[j][q]) + v1[j][q];
+      }
+      // a lane owns row (l % 32) of each 32x32 block and columns 8q + 4(l/32) .. +3
+      const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+          const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * (uint32_t)CE : kOutOfRange;
+          if constexpr (ACC_F32) {
+            const f32x4 old = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rc, off, 0, 0));
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, old + sum[j][q]), rc, off, 0, 0);
+          } else {
+            __builtin_amdgcn_raw_buffer_store_b64(
+                round4<DT>(sum[j][q][0], sum[j][q][1], sum[j][q][2], sum[j][q][3]), rc, off, 0, kStoreStreaming);
+          }
+        }
+    }
+  }
 #endif  // __HIP_DEVICE_COMPILE__
 }
 

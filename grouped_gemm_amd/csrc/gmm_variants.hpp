@@ -1,0 +1,38 @@
+// What the host side (gmm_api.hip) and the kernel translation units (gmm_variant.hip) share:
+// tile shapes, epilogue kinds and the table entry through which a variant is prepared and launched.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "gmm_kernel.hpp"
+
+namespace gg {
+
+constexpr int BK = 64, STAGES = 2;
+
+// Tile shapes.  Wide: 256 x 256 outputs per workgroup, 2 x 2 waves of 128 x 128.  Short: 128 x 256,
+// 1 x 4 waves of 128 x 64, for calls whose groups average few rows: with at most 128 rows per
+// group all four waves then share the rows instead of two of them idling (measured 4-7 % faster
+// below about 100 rows per group, slower from 128 on).  The weight-gradient layout always uses the
+// wide shape: its ragged dimension is the depth, not the rows.
+struct Wide {
+  static constexpr int kId = 0, BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2;
+};
+struct Short {
+  static constexpr int kId = 1, BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
+};
+
+enum : int {
+  kEpiStore = 0,    // c in the operands' element type, overwritten
+  kEpiAccF32 = 1,   // c in fp32, added to (weight-gradient layout only)
+};
+
+struct VariantOps {
+  int dt, layout, shape, epilogue;
+  int lds_bytes;
+  // raises the kernel's dynamic LDS limit on the current device
+  hipError_t (*prepare)();
+  hipError_t (*launch)(const GmmParams& p, const HostSizes& hs, int grid, hipStream_t stream);
+};
+
+}  // namespace gg

@@ -10,6 +10,10 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/extension.h>
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "../../include/grouped_gemm_hip.h"
 
 namespace grouped_gemm {
@@ -29,18 +33,20 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
   TORCH_CHECK(batch_sizes.ndimension() == 1, "grouped_gemm: batch_sizes must be 1-d");
   TORCH_CHECK(batch_sizes.scalar_type() == torch::kInt64, "grouped_gemm: batch_sizes must be int64");
 
-  // a: (tokens, hidden_in) bf16 on the GPU (csrc/grouped_gemm.cu:490-492).
+  // a: (tokens, hidden_in) bf16 on the GPU (csrc/grouped_gemm.cu:490-492).  float16 is accepted
+  // as well, for all three tensors alike; the reference takes bfloat16 only.
   if (on_device) TORCH_CHECK(a.is_cuda(), "grouped_gemm: a must be a GPU tensor");
   TORCH_CHECK(a.ndimension() == 2, "grouped_gemm: a must be 2-d");
-  TORCH_CHECK(a.scalar_type() == torch::kBFloat16, "grouped_gemm: a must be bfloat16");
+  TORCH_CHECK(a.scalar_type() == torch::kBFloat16 || a.scalar_type() == torch::kFloat16,
+              "grouped_gemm: a must be bfloat16 (or float16)");
 
   // b, c: bf16 on the GPU (csrc/grouped_gemm.cu:503-506).
   if (on_device) {
     TORCH_CHECK(b.is_cuda(), "grouped_gemm: b must be a GPU tensor");
     TORCH_CHECK(c.is_cuda(), "grouped_gemm: c must be a GPU tensor");
   }
-  TORCH_CHECK(b.scalar_type() == torch::kBFloat16, "grouped_gemm: b must be bfloat16");
-  TORCH_CHECK(c.scalar_type() == torch::kBFloat16, "grouped_gemm: c must be bfloat16");
+  TORCH_CHECK(b.scalar_type() == a.scalar_type(), "grouped_gemm: b must be bfloat16 (the element type of a)");
+  TORCH_CHECK(c.scalar_type() == a.scalar_type(), "grouped_gemm: c must be bfloat16 (the element type of a)");
 
   if (trans_a) {
     // b (tokens, hidden_out), c (num_experts, hidden_in, hidden_out)
@@ -71,11 +77,9 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
   TORCH_CHECK(b.is_contiguous(), "grouped_gemm: b must be contiguous");
   TORCH_CHECK(c.is_contiguous(), "grouped_gemm: c must be contiguous");
 
-  // Device-resident sizes are scheduled by one launch (csrc/grouped_gemm.cu:120-124).
+  // Device-resident sizes: any number of experts (the reference stops at 512,
+  // csrc/grouped_gemm.cu:120-124; here further experts go to further launches).
   if (batch_sizes.is_cuda()) {
-    TORCH_CHECK(batch_sizes.size(0) <= GG_MAX_GROUPS_PER_LAUNCH, "At most ", GG_MAX_GROUPS_PER_LAUNCH,
-                " experts are supported when batch_sizes is a GPU tensor, but got ",
-                batch_sizes.size(0));
     TORCH_CHECK(batch_sizes.is_contiguous(), "grouped_gemm: batch_sizes must be contiguous");
     if (on_device)
       TORCH_CHECK(batch_sizes.device() == a.device(), "grouped_gemm: batch_sizes is on another GPU");
@@ -86,30 +90,72 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
   }
 }
 
+// Workspace for the depth pieces of a call's last round (see gg_gmm): one per device and stream,
+// allocated and zeroed at the first call there and kept for the life of the process.  Calls on one
+// stream run one after the other, so they can share it; the kernels leave its counters zero.
+torch::Tensor Workspace(const torch::Device& device, hipStream_t stream) {
+  static std::mutex mu;
+  static std::map<std::pair<int, hipStream_t>, torch::Tensor> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  auto key = std::make_pair((int)device.index(), stream);
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    torch::Tensor ws = torch::zeros({(int64_t)GG_WORKSPACE_BYTES}, torch::dtype(torch::kUInt8).device(device));
+    it = cache.emplace(key, ws).first;
+  }
+  return it->second;
+}
+
+void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c, const torch::Tensor& batch_sizes,
+         bool trans_a, bool trans_b, bool accumulate_f32, int64_t flags) {
+  torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
+  TORCH_CHECK(gg_init() == GG_OK, "grouped_gemm: ", gg_last_error());
+  torch::Tensor ws = Workspace(a.device(), stream);
+  gg_gmm_args g = {};
+  g.struct_bytes = sizeof(g);
+  g.dtype = a.scalar_type() == torch::kFloat16 ? GG_DTYPE_F16 : GG_DTYPE_BF16;
+  g.a = a.data_ptr();
+  g.b = b.data_ptr();
+  g.c = c.data_ptr();
+  g.batch_sizes = sizes.data_ptr<int64_t>();
+  g.batch_sizes_on_device = sizes.is_cuda() ? 1 : 0;
+  g.trans_a = trans_a ? 1 : 0;
+  g.trans_b = trans_b ? 1 : 0;
+  g.accumulate_f32 = accumulate_f32 ? 1 : 0;
+  g.num_groups = sizes.size(0);
+  g.tokens = a.size(0);
+  g.hidden_in = a.size(1);
+  g.hidden_out = trans_a ? b.size(1) : (trans_b ? b.size(1) : b.size(2));
+  g.workspace = ws.data_ptr();
+  g.workspace_bytes = (uint64_t)ws.numel();
+  g.flags = (int32_t)flags;
+  g.stream = static_cast<void*>(stream);
+  const int rc = gg_gmm(&g);
+  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+}
+
 }  // namespace
 
 void GroupedGemm(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes,
                  bool trans_a, bool trans_b) {
   Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/true);
+  Run(a, b, c, batch_sizes, trans_a, trans_b, /*accumulate_f32=*/false, /*flags=*/0);
+}
 
-  const int64_t tokens = a.size(0);
-  const int64_t hidden_in = a.size(1);
-  const int64_t hidden_out = trans_a ? b.size(1) : (trans_b ? b.size(1) : b.size(2));
-  torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
-
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
-  const int rc = gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), sizes.data_ptr<int64_t>(),
-                             sizes.is_cuda() ? 1 : 0, sizes.size(0), tokens, hidden_in, hidden_out,
-                             trans_a ? 1 : 0, trans_b ? 1 : 0, static_cast<void*>(stream));
-  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+// gmm with GG_FLAG_* bits, for tests that compare the ways a call can be scheduled.
+void GroupedGemmWithFlags(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes,
+                          bool trans_a, bool trans_b, int64_t flags) {
+  Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/true);
+  Run(a, b, c, batch_sizes, trans_a, trans_b, /*accumulate_f32=*/false, flags);
 }
 
 // c (num_experts, hidden_in, hidden_out) fp32 += per expert a_e^T @ b_e; see gg_gmm_bf16_acc_f32.
 void AccumulateWeightGradient(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes) {
   TORCH_CHECK(c.scalar_type() == torch::kFloat32, "grouped_gemm: the accumulated gradient must be float32");
   // every other check is the one of the bf16 weight-gradient call
-  torch::Tensor shape_of_c = torch::empty(c.sizes(), torch::dtype(torch::kBFloat16).device(torch::kMeta));
+  torch::Tensor shape_of_c = torch::empty(c.sizes(), torch::dtype(a.scalar_type()).device(torch::kMeta));
   Validate(a, b, shape_of_c, batch_sizes, /*trans_a=*/true, /*trans_b=*/false, /*on_device=*/false);
   TORCH_CHECK(a.is_cuda() && b.is_cuda() && c.is_cuda(), "grouped_gemm: a, b and c must be GPU tensors");
   TORCH_CHECK(b.device() == a.device() && c.device() == a.device(),
@@ -117,13 +163,7 @@ void AccumulateWeightGradient(torch::Tensor a, torch::Tensor b, torch::Tensor c,
   TORCH_CHECK(c.is_contiguous(), "grouped_gemm: c must be contiguous");
   if (batch_sizes.is_cuda())
     TORCH_CHECK(batch_sizes.device() == a.device(), "grouped_gemm: batch_sizes is on another GPU");
-  torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
-  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
-  const int rc = gg_gmm_bf16_acc_f32(a.data_ptr(), b.data_ptr(), c.data_ptr<float>(),
-                                     sizes.data_ptr<int64_t>(), sizes.is_cuda() ? 1 : 0, sizes.size(0),
-                                     a.size(0), a.size(1), b.size(1), static_cast<void*>(stream));
-  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+  Run(a, b, c, batch_sizes, /*trans_a=*/true, /*trans_b=*/false, /*accumulate_f32=*/true, /*flags=*/0);
 }
 
 // The on-device scheduler's view of the groups, as an int64 tensor
@@ -151,6 +191,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         [](torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes, bool trans_a,
            bool trans_b) { Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/false); },
         "Shape, rank and dtype checks of gmm without the device checks.");
+  m.def("gmm_with_flags", &GroupedGemmWithFlags, "gmm with GG_FLAG_* bits (testing).");
+  m.attr("flag_whole_tiles") = GG_FLAG_WHOLE_TILES;
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,
         "c (fp32) += per expert a_e^T @ b_e.");
   m.def("debug_schedule", &DebugSchedule, "Per-group table derived by the on-device scheduler.");

@@ -46,40 +46,50 @@ def gmm(a, b, batch_sizes, trans_b=False):
 # the reference's surface (its ops.py stops at gmm above); results and gradients are those of
 # GroupedGemm, through the same backend calls.
 
-@torch.library.custom_op("grouped_gemm_amd::gmm", mutates_args=())
-def _gmm_op(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_a: bool,
-            trans_b: bool) -> torch.Tensor:
-    return backend.gmm(a, b, batch_sizes, trans_a=trans_a, trans_b=trans_b)
+def _register_traceable():
+    @torch.library.custom_op("grouped_gemm_amd::gmm", mutates_args=())
+    def _gmm_op(a: torch.Tensor, b: torch.Tensor, batch_sizes: torch.Tensor, trans_a: bool,
+                trans_b: bool) -> torch.Tensor:
+        return backend.gmm(a, b, batch_sizes, trans_a=trans_a, trans_b=trans_b)
+
+    @_gmm_op.register_fake
+    def _gmm_op_fake(a, b, batch_sizes, trans_a, trans_b):
+        return backend._allocate_output(a, b, batch_sizes, trans_a, trans_b)
+
+    def _gmm_op_setup_context(ctx, inputs, output):
+        a, b, batch_sizes, trans_a, trans_b = inputs
+        if trans_a:   # only reached when a gradient is wanted
+            raise RuntimeError("grouped_gemm_amd::gmm is differentiable as a @ b or a @ b^T only "
+                               "(trans_a=False), as GroupedGemm is")
+        ctx.save_for_backward(a, b, batch_sizes)
+        ctx.trans_b = trans_b
+
+    def _gmm_op_backward(ctx, grad):
+        grad = grad.contiguous()
+        a, b, batch_sizes = ctx.saved_tensors
+        agrad = bgrad = None
+        if ctx.needs_input_grad[0]:
+            agrad = _gmm_op(grad, b, batch_sizes, False, not ctx.trans_b)
+        if ctx.needs_input_grad[1]:
+            lhs, rhs = (grad, a) if ctx.trans_b else (a, grad)
+            bgrad = _gmm_op(lhs, rhs, batch_sizes, True, False)
+        return agrad, bgrad, None, None, None
+
+    torch.library.register_autograd("grouped_gemm_amd::gmm", _gmm_op_backward,
+                                    setup_context=_gmm_op_setup_context)
+    return _gmm_op
 
 
-@_gmm_op.register_fake
-def _gmm_op_fake(a, b, batch_sizes, trans_a, trans_b):
-    return backend._allocate_output(a, b, batch_sizes, trans_a, trans_b)
-
-
-def _gmm_op_setup_context(ctx, inputs, output):
-    a, b, batch_sizes, trans_a, trans_b = inputs
-    assert not trans_a, "the differentiable form is a @ b or a @ b^T, as in GroupedGemm"
-    ctx.save_for_backward(a, b, batch_sizes)
-    ctx.trans_b = trans_b
-
-
-def _gmm_op_backward(ctx, grad):
-    grad = grad.contiguous()
-    a, b, batch_sizes = ctx.saved_tensors
-    agrad = bgrad = None
-    if ctx.needs_input_grad[0]:
-        agrad = _gmm_op(grad, b, batch_sizes, False, not ctx.trans_b)
-    if ctx.needs_input_grad[1]:
-        lhs, rhs = (grad, a) if ctx.trans_b else (a, grad)
-        bgrad = _gmm_op(lhs, rhs, batch_sizes, True, False)
-    return agrad, bgrad, None, None, None
-
-
-torch.library.register_autograd("grouped_gemm_amd::gmm", _gmm_op_backward,
-                                setup_context=_gmm_op_setup_context)
+# torch.library.custom_op exists from PyTorch 2.4 on; the reference's surface above must import
+# on older versions too, so only gmm_traceable depends on it.
+try:
+    _gmm_op = _register_traceable()
+except AttributeError:  # pragma: no cover - depends on the installed PyTorch
+    _gmm_op = None
 
 
 def gmm_traceable(a, b, batch_sizes, trans_b=False):
     """gmm for code that goes through torch.compile: same results and gradients as gmm."""
+    if _gmm_op is None:
+        raise RuntimeError("gmm_traceable needs torch.library.custom_op (PyTorch 2.4 or newer)")
     return _gmm_op(a, b, batch_sizes, False, trans_b)

@@ -9,7 +9,7 @@
  * gg_gmm_bf16.
  *
  * All functions return 0 on success and a negative GG_E* code on failure;
- * gg_last_error() then holds a message for the calling thread.  Nothing here
+ * gg_last_error() then holds a message for the calling thread.  No entry point
  * synchronises the device or allocates device memory.
  */
 #ifndef GROUPED_GEMM_HIP_H_
@@ -23,17 +23,40 @@ extern "C" {
 
 #define GG_OK 0
 #define GG_EINVAL (-1)   /* bad argument (null pointer, negative size, both transposes, ...) */
-#define GG_ELIMIT (-2)   /* a documented limit is exceeded (alignment, group count, 32-bit ranges) */
+#define GG_ELIMIT (-2)   /* a documented limit is exceeded (alignment, 32-bit ranges, workspace) */
 #define GG_EHIP (-3)     /* a HIP runtime call failed */
 
 /* Most groups one launch schedules on the device.  Same value as the reference's
  * kMaxExperts (csrc/fill_arguments.cuh:11, enforced at csrc/grouped_gemm.cu:120-124).
- * Host-resident batch_sizes with more groups are split into several launches. */
+ * Calls with more groups are split into several launches, whether batch_sizes lives on the
+ * host or on the device (the reference rejects the latter). */
 #define GG_MAX_GROUPS_PER_LAUNCH 512
 
-/* Columns of one row of the table written by gg_debug_schedule. */
-#define GG_SCHED_COLS 12
-/* m, n, k, lda, ldb, ldc, a_off, b_off, c_off (elements), first_tile, num_tiles, rows_used */
+/* Columns of one row of the table written by gg_debug_schedule:
+ * m, n, k, lda, ldb, ldc, a_off, b_off, c_off (elements), first_tile, num_tiles, rows_used,
+ * first_runt_tile, num_runt_tiles. */
+#define GG_SCHED_COLS 14
+
+/* Element types of a and b (and of c, unless it is the fp32 accumulator). */
+#define GG_DTYPE_BF16 0
+#define GG_DTYPE_F16 1
+
+/* Bytes of workspace that let any call cut the tiles of its last, partly filled round along the
+ * depth (see gg_gmm): 4096 bytes of arrival counters and 256 partial tiles of 256 x 256 floats. */
+#define GG_WORKSPACE_BYTES (4096 + 256 * 256 * 256 * 4)
+
+/* gg_gmm_args.flags: debugging switches, for comparing the ways a call can be scheduled.  None
+ * changes what is computed; results agree to within fp32 summation order. */
+#define GG_FLAG_WHOLE_TILES 1   /* never cut the tiles of the last round into pieces */
+#define GG_FLAG_ONE_CLASS 2     /* hand out a tall group's short last tile row in place, not after all other tiles */
+#define GG_FLAG_ROW_PIECES 4    /* ignore the workspace: cut the last round's tiles along the rows only */
+
+/*
+ * One-time set-up for the current device: checks that it is a gfx950 and raises the LDS limit
+ * of every kernel variant.  Every other entry point does the same on its first call on a
+ * device; call this first where that first call must not happen inside a HIP graph capture.
+ */
+int gg_init(void);
 
 /*
  * Grouped GEMM, bf16 in, fp32 accumulate, bf16 out, alpha = 1, beta = 0.
@@ -54,14 +77,17 @@ extern "C" {
  * a group is overwritten; rows of c past sum(batch_sizes) are not touched.
  * batch_sizes: int64[num_groups], in host memory (batch_sizes_on_device = 0) or device
  * memory (1).  Device-resident sizes are read by the kernel itself; the host never
- * waits for them.  Rows a group would take past `tokens` are ignored, so no size
- * vector can make the kernel read or write outside a, b or c.
+ * waits for them.  Each size is clamped to [0, tokens] and rows a group would take past
+ * `tokens` are ignored, so no size vector can make the kernel read or write outside a, b or c.
+ * Host-resident sizes that are negative or sum past `tokens` are rejected (GG_EINVAL).
  * stream: a hipStream_t (NULL = the default stream).
+ *
+ * One persistent launch (one per 512 groups).  Uses no workspace: the tiles of a partly filled
+ * last round are cut along their rows only; gg_gmm with a workspace cuts them along the depth.
  *
  * Limits (GG_ELIMIT): a, b and c 16-byte aligned, hidden_in and hidden_out multiples of 8
  * (16-byte rows, the same alignment the reference's kernel configuration assumes,
- * csrc/grouped_gemm.cu:41-66) and below 2^22; tokens below 2^31; num_groups <= GG_MAX_GROUPS_PER_LAUNCH when
- * batch_sizes is on the device.
+ * csrc/grouped_gemm.cu:41-66) and below 2^22; tokens below 2^31.
  */
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,
                 int batch_sizes_on_device, int64_t num_groups, int64_t tokens,
@@ -85,14 +111,60 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
                         int64_t hidden_in, int64_t hidden_out, void* stream);
 
 /*
+ * The general form: everything gg_gmm_bf16 and gg_gmm_bf16_acc_f32 do, selected by fields, plus
+ * what the reference's entry point (csrc/grouped_gemm.cu:470-564) has no argument for.  Zero
+ * the struct, set struct_bytes = sizeof(gg_gmm_args), fill in what is needed.
+ *
+ *   dtype         GG_DTYPE_BF16 or GG_DTYPE_F16: element type of a, b and c (the reference
+ *                 rejects everything but bf16, csrc/grouped_gemm.cu:492, 505-506).
+ *   accumulate_f32  1: c is fp32 and is added to (trans_a = 1 only), as gg_gmm_bf16_acc_f32.
+ *   workspace, workspace_bytes
+ *                 Device memory the call may use for partial results, or NULL.  When the last
+ *                 round of the persistent grid is at most half full, each of its tiles is cut
+ *                 into 2 to 8 pieces along the depth; a piece adds up its depth slices into an
+ *                 fp32 partial tile in the workspace, and the piece that finishes last sums the
+ *                 partial tiles in piece order and stores the result, so the output does not
+ *                 depend on timing.  The first 4096 bytes (arrival counters) must be zero
+ *                 before the first call and are zero again after every call; the rest needs no
+ *                 initialisation.  GG_WORKSPACE_BYTES serves every call; a smaller workspace
+ *                 (at least 4096 + one 256 KiB tile) serves fewer pieces; 256-byte aligned.
+ *                 Calls that share a workspace must not overlap in time (same stream is enough).
+ *   flags         GG_FLAG_* bits.
+ */
+typedef struct gg_gmm_args {
+  uint32_t struct_bytes;
+  int32_t dtype;
+  const void* a;
+  const void* b;
+  void* c;
+  const int64_t* batch_sizes;
+  int32_t batch_sizes_on_device;
+  int32_t trans_a;
+  int32_t trans_b;
+  int32_t accumulate_f32;
+  int64_t num_groups;
+  int64_t tokens;
+  int64_t hidden_in;
+  int64_t hidden_out;
+  void* workspace;
+  uint64_t workspace_bytes;
+  int32_t flags;
+  int32_t reserved0;
+  void* stream;
+} gg_gmm_args;
+
+int gg_gmm(const gg_gmm_args* args);
+
+/*
  * Runs only the on-device scheduler of gg_gmm_bf16 (same device code, same
  * arguments) and writes what it derived to `table_out`, a device buffer of
  * num_groups * GG_SCHED_COLS int64: per group the problem (m, n, k), leading
  * dimensions, element offsets of its A, B and C blocks, its first tile index, its tile
- * count and the rows of `a` it uses.  The first nine columns are the quantities of
- * the reference's problem table (csrc/fill_arguments.cuh:63-78,
- * csrc/grouped_gemm.cu:159-175) and must equal its int64 closed forms bit for bit.
- * num_groups <= GG_MAX_GROUPS_PER_LAUNCH.
+ * count, the rows of `a` it uses, and the first index and count of its tiles of the second
+ * class (the much shorter last tile row of a tall group, handed out after all other tiles).
+ * The first nine columns are the quantities of the reference's problem table
+ * (csrc/fill_arguments.cuh:63-78, csrc/grouped_gemm.cu:159-175) and must equal its int64
+ * closed forms bit for bit.  num_groups <= GG_MAX_GROUPS_PER_LAUNCH.
  */
 int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device,
                       int64_t num_groups, int64_t tokens, int64_t hidden_in,

@@ -22,7 +22,8 @@ Contents
                       operator-precedence quirk included.
   allclose_ops_test   the reference tests' own acceptance rule (ops_test.py:10-17).
   assert_close_bf16   this build's acceptance rule: every element within
-                      rtol 1.6e-2, atol 1e-2 of the fp32-accumulated oracle.
+                      rtol 1.6e-2, atol 1e-2 of the fp32-accumulated oracle, the absolute
+                      term scaled down to the output's root-mean-square where that is below 1.
 
 Pinned in tests/test_oracle.py; no function here is "parity unpinned".
 """
@@ -220,19 +221,31 @@ def allclose_ops_test(x, y, pct=2.0):
     return pct_diff <= pct
 
 
+def atol_for(want_fp32, atol=ATOL):
+    """The absolute term of the tolerance, scaled to the data: `atol` where the expected output
+    has unit scale or more, `atol` times its root-mean-square where it is smaller, so that an
+    output of small numbers cannot pass by being small (an all-zero answer against expected
+    values of a few thousandths, say)."""
+    want = want_fp32.float()
+    if want.numel() == 0:
+        return atol
+    rms = float(want.double().pow(2).mean().sqrt())
+    return atol * min(1.0, rms)
+
+
 def max_violation(got, want_fp32, rtol=RTOL, atol=ATOL):
-    """max over elements of |got-want| - (atol + rtol*|want|); <= 0 means pass."""
+    """max over elements of |got-want| - (atol_for(want) + rtol*|want|); <= 0 means pass."""
     got = got.float()
     want = want_fp32.float()
     if got.numel() == 0:
         return 0.0
-    return float(((got - want).abs() - (atol + rtol * want.abs())).max())
+    return float(((got - want).abs() - (atol_for(want, atol) + rtol * want.abs())).max())
 
 
 def assert_close_bf16(got, want_fp32, rtol=RTOL, atol=ATOL, what=""):
     assert tuple(got.shape) == tuple(want_fp32.shape), (what, got.shape, want_fp32.shape)
     v = max_violation(got, want_fp32, rtol, atol)
-    assert v <= 0.0, f"{what}: element outside rtol={rtol} atol={atol} by {v}"
+    assert v <= 0.0, f"{what}: element outside rtol={rtol} atol={atol} (scaled to the data) by {v}"
 
 
 def cpu_loop_bf16(a, b, batch_sizes, trans_a=False, trans_b=False):

@@ -5,10 +5,11 @@ fixed sizes, variable sizes, the zero-size expert at Mixtral shape, the zero-K k
 answer; then the five benchmark configurations, the C ABI called directly, the
 on-device schedule bit-exact against the int64 closed forms, and edge cases.
 
-Tolerance (every element): |got - want| <= 1e-2 + 1.6e-2 * |want| against the
-fp32-accumulated oracle.  Small cases use the oracle on the CPU; full-size cases run
-the oracle's per-expert loop with torch on the GPU in fp32 and add a CPU fp64 check on
-sampled rows so that no GPU library is trusted alone.
+Tolerance (every element): |got - want| <= 1e-2 * min(1, rms(want)) + 1.6e-2 * |want| against
+the fp32-accumulated oracle: the absolute term is scaled down to the data, so outputs of small
+numbers cannot pass by being small.  Small cases use the oracle on the CPU; full-size cases run
+the oracle's per-expert loop with torch on the GPU in fp32 and add CPU fp64 checks on
+sampled rows and entries so that no GPU library is trusted alone.
 """
 import ctypes
 import os
@@ -40,8 +41,15 @@ def check(got, want, what):
     assert tuple(got.shape) == tuple(want.shape), (what, got.shape, want.shape)
     if got.numel() == 0:
         return
-    viol = float(((got - want).abs() - (ATOL + RTOL * want.abs())).max())
-    assert viol <= 0.0, f"{what}: outside rtol={RTOL} atol={ATOL} by {viol}"
+    atol = ATOL * min(1.0, float(want.double().pow(2).mean().sqrt()))
+    viol = float(((got - want).abs() - (atol + RTOL * want.abs())).max())
+    assert viol <= 0.0, f"{what}: outside rtol={RTOL} atol={atol} by {viol}"
+
+
+def _gmm_flags(ops, a, b, bs, flags, trans_a=False, trans_b=False):
+    c = ops.backend._allocate_output(a, b, bs, trans_a, trans_b)
+    ops.backend.backend.gmm_with_flags(a, b, c, bs, trans_a, trans_b, flags)
+    return c
 
 
 def fp64_rows_check(a, b, sizes, trans_b, out, nrows=24, seed=0):
@@ -58,6 +66,22 @@ def fp64_rows_check(a, b, sizes, trans_b, out, nrows=24, seed=0):
         w = b[e].double().cpu()
         want = a[r].double().cpu() @ (w.t() if trans_b else w)
         check(out[r].cpu(), want, f"fp64 row {r} of expert {e}")
+
+
+def fp64_weight_gradient_check(lhs, rhs, sizes, bgrad, nblocks=12, seed=2):
+    """CPU float64 recomputation of 16 x 16 blocks of the weight gradient of sampled experts
+    (first, last and random rows and columns): lhs_e^T @ rhs_e, independent of any GPU library."""
+    g = torch.Generator().manual_seed(seed)
+    starts = torch.cumsum(sizes, 0) - sizes
+    hin, hout = lhs.shape[1], rhs.shape[1]
+    for n in range(nblocks):
+        e = int(torch.randint(len(sizes), (1,), generator=g))
+        s, m = int(starts[e]), int(sizes[e])
+        i0 = [0, hin - 16, int(torch.randint(hin - 15, (1,), generator=g))][n % 3]
+        j0 = [hout - 16, 0, int(torch.randint(hout - 15, (1,), generator=g))][n % 3]
+        want = lhs[s:s + m, i0:i0 + 16].double().cpu().t() @ rhs[s:s + m, j0:j0 + 16].double().cpu()
+        got = bgrad[e, i0:i0 + 16, j0:j0 + 16].cpu()
+        check(got, want, f"fp64 weight gradient block ({i0}, {j0}) of expert {e}")
 
 
 # ------------------------------------------------ mirrors of the reference's tests
@@ -234,6 +258,7 @@ def _full_size_case(ops, oracle, config):
                 s, m = int(starts[e]), int(sizes[e])
                 want = lhs[s:s + m].float().t() @ rhs[s:s + m].float()
                 check(bg[e], want, f"bgrad expert {e}")
+            fp64_weight_gradient_check(lhs, rhs, sizes, bg)
             # host-resident sizes must give the very same bits as device-resident ones
             bg2 = ops.backend.gmm(lhs, rhs, sizes, trans_a=True)
             assert torch.equal(bg, bg2)
@@ -252,12 +277,19 @@ def test_config3_ragged_full_size(ops, oracle):
     _announce("config3 full")
     w, res = _full_size_case(ops, oracle, 3)
     assert int((w.batch_sizes == 0).sum()) >= 4
-    # each expert on its own (one group per call) gives the same bits as the grouped call
+    # each expert on its own (one group per call) gives the same bits as the grouped call when
+    # both keep their tiles whole (the depth order of every output element is then the same);
+    # with the last round cut along the depth the two differ by fp32 summation order only
     starts = torch.cumsum(w.batch_sizes, 0) - w.batch_sizes
+    whole_flag = ops.backend.backend.flag_whole_tiles
+    grouped_whole = _gmm_flags(ops, w.a, w.b, w.batch_sizes.cuda(), whole_flag)
+    check(grouped_whole, res["fwd"].float(), "whole tiles against depth pieces")
     for e in [int(torch.argmax(w.batch_sizes)), int(torch.argmin(w.batch_sizes + (w.batch_sizes == 0) * 10 ** 9))]:
         s, m = int(starts[e]), int(w.batch_sizes[e])
-        alone = ops.backend.gmm(w.a[s:s + m].contiguous(), w.b[e:e + 1].contiguous(), torch.tensor([m]))
-        assert torch.equal(alone, res["fwd"][s:s + m])
+        a_e, b_e = w.a[s:s + m].contiguous(), w.b[e:e + 1].contiguous()
+        alone = _gmm_flags(ops, a_e, b_e, torch.tensor([m]), whole_flag)
+        assert torch.equal(alone, grouped_whole[s:s + m])
+        check(ops.backend.gmm(a_e, b_e, torch.tensor([m])), alone.float(), f"expert {e} alone, depth pieces")
 
 
 def test_config4_weight_gradient_full_size(ops, oracle):
@@ -282,6 +314,7 @@ def test_config5_deepseek_share_full_size_autograd(ops, oracle):
             s, m = int(starts[e]), int(sizes[e])
             want = w.grad[s:s + m].float().t() @ w.a.detach()[s:s + m].float()
             check(b.grad[e], want, f"bgrad expert {e}")
+        fp64_weight_gradient_check(w.grad, w.a.detach(), sizes, b.grad)
         fp64_rows_check(w.a.detach(), w.b.detach(), sizes, True, out.detach())
 
 
@@ -358,26 +391,59 @@ def test_every_row_block_count(ops, oracle, trans_b, on_device):
     assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("trans_b", [False, True])
-def test_last_round_pieces_equal_whole_tiles(ops, oracle, trans_b, monkeypatch):
-    # A launch with fewer tiles than workgroups cuts its tiles into row pieces for the idle
-    # workgroups; GG_TAIL_SPLIT=0 keeps them whole.  Same depth order per output element either
-    # way, so the two must agree bit for bit (and with the oracle within tolerance).
-    for idx, (sizes, hin, hout) in enumerate(_random_cases(16, seed=91 + int(trans_b))):
-        _announce("pieces", trans_b, sizes, hin, hout)
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_last_round_pieces_against_whole_tiles(ops, oracle, layout):
+    # A launch with fewer tiles than workgroups cuts its tiles into pieces for the idle
+    # workgroups (along the depth, summed through the workspace in a fixed order); the flag keeps
+    # them whole.  The two differ only in the order of fp32 additions: both must match the oracle,
+    # agree with each other far inside the tolerance, and each be the same bits on every call.
+    trans_a, trans_b = layout
+    whole_flag = ops.backend.backend.flag_whole_tiles
+    for idx, (sizes, hin, hout) in enumerate(_random_cases(16, seed=91 + int(trans_b) + 2 * int(trans_a))):
+        hin = hin * 8 if idx % 2 else hin     # deep enough for several depth pieces
+        _announce("pieces", layout, sizes, hin, hout)
         g = torch.Generator().manual_seed(idx)
         bs = torch.tensor(sizes, dtype=torch.int64)
         t = int(bs.sum())
         a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
-        b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16).cuda()
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(torch.bfloat16).cuda()
+        else:
+            b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16).cuda()
         dev_bs = bs.cuda() if idx % 2 else bs
-        monkeypatch.setenv("GG_TAIL_SPLIT", "1")
-        cut = ops.backend.gmm(a, b, dev_bs, trans_b=trans_b)
-        monkeypatch.setenv("GG_TAIL_SPLIT", "0")
-        whole = ops.backend.gmm(a, b, dev_bs, trans_b=trans_b)
-        assert torch.equal(cut, whole), f"case {idx}: sizes={sizes} hin={hin} hout={hout}"
-        check(whole, oracle.gmm_loop(a.cpu(), b.cpu(), bs, trans_b=trans_b), f"case {idx}")
-    monkeypatch.delenv("GG_TAIL_SPLIT")
+        cut = _gmm_flags(ops, a, b, dev_bs, 0, trans_a, trans_b)
+        whole = _gmm_flags(ops, a, b, dev_bs, whole_flag, trans_a, trans_b)
+        want = oracle.gmm_loop(a.cpu(), b.cpu(), bs, trans_a=trans_a, trans_b=trans_b)
+        check(whole, want, f"whole, case {idx}")
+        check(cut, want, f"cut, case {idx}")
+        if want.numel():    # one bf16 rounding step apart at most, relative to the largest value
+            assert float((cut.float() - whole.float()).abs().max()) <= 2 ** -7 * float(want.abs().max())
+        assert torch.equal(cut, _gmm_flags(ops, a, b, dev_bs, 0, trans_a, trans_b))
+
+
+def test_c_abi_without_workspace_cuts_rows_bit_exactly(oracle):
+    # gg_gmm_bf16 brings no workspace: the tiles of the last round are cut along their rows, which
+    # leaves the depth order of every output element alone, so the result equals the whole-tile
+    # one bit for bit.
+    lib = _c_abi()
+    whole_flag = 1
+    for idx, (sizes, hin, hout) in enumerate(_random_cases(8, seed=77)):
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
+        b = torch.randn(len(sizes), hin, hout, generator=g).to(torch.bfloat16).cuda()
+        c1 = torch.zeros(t, hout, dtype=torch.bfloat16, device="cuda")
+        c2 = torch.zeros_like(c1)
+        _announce("row pieces", sizes, hin, hout)
+        rc = lib.gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c1.data_ptr(), bs.data_ptr(), 0, len(sizes), t, hin, hout,
+                             0, 0, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.gg_last_error()
+        args = _gmm_args(lib, a, b, c2, bs, False, t, hin, hout, 0, 0, flags=whole_flag)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(c1, c2)
+        check(c1, oracle.gmm_loop(a.cpu(), b.cpu(), bs), f"case {idx}")
 
 
 # ----------------------------------------------------------------- schedule, bit-exact
@@ -404,8 +470,11 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
     want = oracle.table_closed(sizes, hin, hout, trans_a, trans_b)
     np.testing.assert_array_equal(got[:, :9], want)
     assert np.array_equal(want, oracle.table_walk(sizes, hin, hout, trans_a, trans_b)[0])
-    # tiles: consecutive, non-overlapping, and enough to cover each group's output
-    assert np.array_equal(got[:, 9], np.cumsum(got[:, 10]) - got[:, 10])
+    # tiles: two classes (all tiles but the runt rows, then the runt rows), each consecutive and
+    # non-overlapping, together enough to cover each group's output
+    first_class = got[:, 10] - got[:, 13]
+    assert np.array_equal(got[:, 9], np.cumsum(first_class) - first_class)
+    assert np.array_equal(got[:, 12], first_class.sum() + np.cumsum(got[:, 13]) - got[:, 13])
     assert np.array_equal(got[:, 11], np.array(sizes))
     lib = ctypes.CDLL(os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so"))
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
@@ -413,6 +482,17 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
                       ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk))
     m, n = got[:, 0], got[:, 1]
     assert np.array_equal(got[:, 10], -(-m // bm.value) * -(-n // bn.value))
+    # a runt row is the last tile row of a group of at least two, at most half as many 32-row
+    # blocks tall as the others
+    if not trans_a:
+        tiles_n = -(-n // bn.value)
+        tiles_m = -(-m // bm.value)
+        height = -(-(-(-m // np.maximum(tiles_m, 1))) // 32) * 32
+        last_blocks = -(-(m - (tiles_m - 1) * height) // 32)
+        runt = (tiles_m >= 2) & (2 * last_blocks <= height // 32)
+        assert np.array_equal(got[:, 13], runt * tiles_n)
+    else:
+        assert not got[:, 13].any()
 
 
 def test_schedule_clips_rows_past_tokens(ops):
@@ -423,6 +503,23 @@ def test_schedule_clips_rows_past_tokens(ops):
     assert got[:, 6].tolist() == [0, 100 * 64, 150 * 64]
 
 
+def test_schedule_saturates_huge_and_negative_sizes(ops):
+    # sizes from an uninitialised buffer: each is clamped to [0, tokens] before it enters a sum, so
+    # no sum wraps, no group starts before row 0 and none reaches past `tokens`
+    big = (1 << 63) - 1
+    for sizes, want_rows, want_start in [
+        ([big, big, 5], [150, 0, 0], [0, 150, 150]),
+        ([-big, 7, big], [0, 7, 143], [0, 0, 7]),
+        ([-1, -(1 << 62), 150, 3], [0, 0, 150, 0], [0, 0, 0, 150]),
+    ]:
+        bs = torch.tensor(sizes, dtype=torch.int64).cuda()
+        for trans_a in (False, True):
+            got = ops.backend.debug_schedule(bs, 150, 64, 64, trans_a, False).cpu().numpy()
+            assert got[:, 11].tolist() == want_rows, (sizes, got[:, 11])
+            assert got[:, 6].tolist() == [s * 64 for s in want_start]
+            assert (got[:, 6:9] >= 0).all()
+
+
 # ----------------------------------------------------------------- C ABI, directly
 
 def _c_abi():
@@ -431,7 +528,36 @@ def _c_abi():
     lib.gg_gmm_bf16.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
                                 ctypes.c_int, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                 ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.gg_gmm.argtypes = [ctypes.c_void_p]
     return lib
+
+
+class GmmArgs(ctypes.Structure):
+    """gg_gmm_args of include/grouped_gemm_hip.h."""
+    _fields_ = [("struct_bytes", ctypes.c_uint32), ("dtype", ctypes.c_int32),
+                ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p),
+                ("batch_sizes", ctypes.c_void_p), ("batch_sizes_on_device", ctypes.c_int32),
+                ("trans_a", ctypes.c_int32), ("trans_b", ctypes.c_int32), ("accumulate_f32", ctypes.c_int32),
+                ("num_groups", ctypes.c_int64), ("tokens", ctypes.c_int64),
+                ("hidden_in", ctypes.c_int64), ("hidden_out", ctypes.c_int64),
+                ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_uint64),
+                ("flags", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("stream", ctypes.c_void_p)]
+
+
+def _gmm_args(lib, a, b, c, sizes, on_device, tokens, hin, hout, trans_a, trans_b, flags=0, workspace=None,
+              dtype=0, stream=None):
+    g = GmmArgs()
+    g.struct_bytes = ctypes.sizeof(GmmArgs)
+    g.dtype = dtype
+    g.a, g.b, g.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+    g.batch_sizes, g.batch_sizes_on_device = sizes.data_ptr(), int(on_device)
+    g.trans_a, g.trans_b = int(trans_a), int(trans_b)
+    g.num_groups, g.tokens, g.hidden_in, g.hidden_out = sizes.numel(), tokens, hin, hout
+    if workspace is not None:
+        g.workspace, g.workspace_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
+    g.flags = flags
+    g.stream = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+    return g
 
 
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
@@ -473,9 +599,35 @@ def test_c_abi_rejects_bad_host_sizes():
         s = torch.tensor(sizes, dtype=torch.int64)
         rc = lib.gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), s.data_ptr(), 0, 2, 16, 8, 8, 0, 0, None)
         assert rc == -1, sizes
-    s = torch.zeros(513, dtype=torch.int64, device="cuda")
-    rc = lib.gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), s.data_ptr(), 1, 513, 16, 8, 8, 0, 0, None)
-    assert rc == -2 and b"512" in lib.gg_last_error()
+    big = (1 << 63) - 1                                        # would wrap a running sum
+    s = torch.tensor([10, big], dtype=torch.int64)
+    rc = lib.gg_gmm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), s.data_ptr(), 0, 2, 16, 8, 8, 0, 0, None)
+    assert rc == -1 and b"sum past" in lib.gg_last_error()
+
+
+def test_c_abi_workspace_sizes(oracle):
+    # the general entry point with workspaces of several sizes: every one gives the oracle's
+    # result; a workspace too small for a single partial tile is rejected
+    lib = _c_abi()
+    g = torch.Generator().manual_seed(9)
+    sizes = torch.tensor([300, 40, 0, 129], dtype=torch.int64)
+    t, hin, hout = int(sizes.sum()), 1024, 264
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
+    b = torch.randn(4, hin, hout, generator=g).to(torch.bfloat16).cuda()
+    want = oracle.gmm_loop(a.cpu(), b.cpu(), sizes)
+    slot = 256 * 256 * 4
+    for nbytes in (4096 + slot, 4096 + 7 * slot + 100, 4096 + 64 * slot, 4096 + 256 * slot):
+        _announce("workspace bytes", nbytes)
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        c = torch.full((t, hout), 7.0, dtype=torch.bfloat16, device="cuda")
+        args = _gmm_args(lib, a, b, c, sizes.cuda(), True, t, hin, hout, 0, 0, workspace=ws)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
+        torch.cuda.synchronize()
+        check(c, want, f"workspace of {nbytes} bytes")
+        assert not ws[:4096].any(), "the arrival counters must be zero again after the call"
+    ws = torch.zeros(4096 + slot - 256, dtype=torch.uint8, device="cuda")
+    args = _gmm_args(lib, a, b, c, sizes.cuda(), True, t, hin, hout, 0, 0, workspace=ws)
+    assert lib.gg_gmm(ctypes.byref(args)) == -2 and b"workspace" in lib.gg_last_error()
 
 
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
@@ -586,6 +738,59 @@ def test_traceable_operator_under_torch_compile(ops, trans_b):
     compiled = run(compiled_fn)
     for x, y in zip(eager, compiled):
         assert torch.equal(x, y)
+
+
+# ------------------------------------------------------------------- float16 operands
+
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_float16_random_shapes(ops, oracle, layout):
+    # same kernels with the fp16 matrix instruction and an fp16 rounding on store; the oracle is
+    # the per-expert loop on fp32-upcast slices (the reference takes bf16 only,
+    # csrc/grouped_gemm.cu:492, 505-506).  fp16 keeps 3 more mantissa bits than bf16, so the bf16
+    # tolerance holds with room to spare; values are kept inside the fp16 range.
+    trans_a, trans_b = layout
+    for idx, (sizes, hin, hout) in enumerate(_random_cases(12, seed=41 + int(trans_a) + 2 * int(trans_b))):
+        _announce("fp16", layout, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(torch.float16)
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(torch.float16)
+        else:
+            b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.float16)
+        dev_bs = bs.cuda() if idx % 2 else bs
+        out = ops.backend.gmm(a.cuda(), b.cuda(), dev_bs, trans_a=trans_a, trans_b=trans_b)
+        assert out.dtype == torch.float16
+        want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
+        check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
+        # tighter: one fp16 rounding of the fp32-accumulated value
+        assert float((out.float().cpu() - want).abs().max()) <= 2 ** -10 * float(want.abs().max()) + 1e-6
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_float16_autograd_and_mixed_dtypes(ops, oracle, trans_b):
+    g = torch.Generator().manual_seed(43)
+    sizes = torch.tensor([300, 0, 17, 195])
+    a = torch.randn(512, 256, generator=g).to(torch.float16)
+    b = torch.randn(4, *((384, 256) if trans_b else (256, 384)), generator=g).to(torch.float16)
+    grad = torch.randn(512, 384, generator=g).to(torch.float16)
+    da, db = a.cuda().requires_grad_(True), b.cuda().requires_grad_(True)
+    out = ops.gmm(da, db, sizes.cuda(), trans_b)
+    out.backward(grad.cuda())
+    want, want_ag, want_bg = oracle.gmm_autograd_loop(a, b, sizes, trans_b, grad)
+    check(out.detach(), want, "forward")
+    check(da.grad, want_ag, "agrad")
+    check(db.grad, want_bg, "bgrad")
+    assert (db.grad[1] == 0).all()
+    with pytest.raises(RuntimeError, match="element type"):
+        ops.backend.gmm(a.cuda(), b.cuda().to(torch.bfloat16), sizes)
+    # fp16 operands, fp32 accumulated weight gradient
+    c0 = torch.randn(4, 256, 384, generator=g)
+    c = c0.clone().cuda()
+    ops.backend.accumulate_weight_gradient(a.cuda(), grad.cuda(), sizes.cuda(), c)
+    want_c = oracle.accumulate_weight_gradient_loop(a, grad, sizes, c0)
+    assert float((c.double().cpu() - want_c).abs().max()) <= 1e-4 * float(want_c.abs().max())
 
 
 # ------------------------------------------------- fp32-accumulated weight gradient
@@ -710,8 +915,34 @@ def test_more_than_512_experts(ops, oracle):
     grad = torch.randn(t, 40, generator=g).to(torch.bfloat16)
     bg = ops.backend.gmm(a.cuda(), grad.cuda(), sizes, trans_a=True)
     check(bg, oracle.gmm_loop(a, grad, sizes, trans_a=True), "bgrad")
-    with pytest.raises(RuntimeError, match="512"):                       # csrc/grouped_gemm.cu:120-124
-        ops.backend.gmm(a.cuda(), b.cuda(), sizes.cuda())
+    # device-resident sizes: the reference stops at 512 experts (csrc/grouped_gemm.cu:120-124);
+    # here every launch after the first sums up the sizes of the groups before it on the device
+    out_dev = ops.backend.gmm(a.cuda(), b.cuda(), sizes.cuda())
+    assert torch.equal(out_dev, out)
+    bg_dev = ops.backend.gmm(a.cuda(), grad.cuda(), sizes.cuda(), trans_a=True)
+    assert torch.equal(bg_dev, bg)
+
+
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_many_experts_device_sizes(ops, oracle, layout):
+    # 1500 experts of 0..40 rows, sizes on the device: three launches, offsets of the later ones
+    # derived in the kernel; equal to the host-resident call bit for bit and to the oracle
+    trans_a, trans_b = layout
+    g = torch.Generator().manual_seed(6)
+    e, hin, hout = 1500, 72, 136
+    sizes = torch.randint(0, 41, (e,), generator=g)
+    sizes[::7] = 0
+    t = int(sizes.sum())
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    if trans_a:
+        b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+    else:
+        b = torch.randn(e, *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+    _announce("1500 experts", layout)
+    dev = ops.backend.gmm(a.cuda(), b.cuda(), sizes.cuda(), trans_a=trans_a, trans_b=trans_b)
+    host = ops.backend.gmm(a.cuda(), b.cuda(), sizes, trans_a=trans_a, trans_b=trans_b)
+    assert torch.equal(dev, host)
+    check(dev, oracle.gmm_loop(a, b, sizes, trans_a=trans_a, trans_b=trans_b), "1500 experts")
 
 
 def test_gpu_validation_errors(ops):

@@ -22,6 +22,18 @@ def bf16(*shape):
 
 # ------------------------------------------------------------------ Python surface
 
+def test_extension_module_imports_top_level_first():
+    # setup.py:35 of the reference installs the extension under the top-level name
+    # grouped_gemm_backend; here it resolves once either package has been imported, whichever
+    # comes first, and torch before it (backend.py:1-3)
+    import subprocess
+    import sys
+    for pkg in ("grouped_gemm", "grouped_gemm_amd"):
+        code = (f"import sys; sys.path.insert(0, {ROOT!r}); import {pkg}; import grouped_gemm_backend as m; "
+                "assert callable(m.gmm)")
+        subprocess.run([sys.executable, "-c", code], check=True)
+
+
 def test_package_layout_matches_reference():
     # grouped_gemm/__init__.py:1-2, ops.py:1, ops_test.py:5,154
     import grouped_gemm
@@ -122,7 +134,8 @@ def _declared_functions():
 
 def test_c_abi_exports_every_declared_symbol():
     names = _declared_functions()
-    assert {"gg_gmm_bf16", "gg_debug_schedule", "gg_last_error", "gg_version", "gg_tile_shape"} <= set(names)
+    assert {"gg_gmm_bf16", "gg_gmm", "gg_init", "gg_gmm_bf16_acc_f32", "gg_debug_schedule", "gg_last_error",
+            "gg_version", "gg_tile_shape"} <= set(names)
     lib = ctypes.CDLL(HIP_LIB)
     for n in names:
         assert hasattr(lib, n), n
@@ -149,6 +162,10 @@ def test_c_abi_argument_errors_need_no_device():
     acc = lib.gg_gmm_bf16_acc_f32(ptr(4096), ptr(8192), ptr(12288), sizes, 0, i64(2), i64(8), i64(1 << 20),
                                   i64(24), None)
     assert acc == -2 and b"2^20" in lib.gg_last_error()
+    # host-resident sizes that would wrap a running sum are rejected one by one, before any device call
+    huge = (i64 * 2)(10, (1 << 63) - 1)
+    rc = lib.gg_gmm_bf16(ptr(4096), ptr(8192), ptr(12288), huge, 0, i64(2), i64(16), i64(16), i64(24), 0, 0, None)
+    assert rc == -1 and b"sum past" in lib.gg_last_error()
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     assert lib.gg_tile_shape(i64(8), i64(32768), 0, 0, ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk)) == 0
     assert (bm.value, bn.value, bk.value) == (256, 256, 64)

@@ -56,6 +56,34 @@ def test_c_loop_matches_library_matmul_tn(oracle):
     torch.testing.assert_close(oracle.gmm_loop(a, b, bs, trans_a=True), c32, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_autograd_loop_matches_c_loops(oracle, trans_b):
+    # gmm_autograd_loop (forward and both gradients by autograd through the per-expert loop) against
+    # the plain-C loops: forward is the NN / NT loop, the input gradient the loop with the opposite
+    # layout of b, the weight gradient the TN loop with the operands in the order ops.py:25 uses
+    k, n = 24, 40
+    a = _rand_bf16(sum(SIZES), k, seed=11)
+    b = _rand_bf16(len(SIZES), n, k, seed=12) if trans_b else _rand_bf16(len(SIZES), k, n, seed=12)
+    grad = _rand_bf16(sum(SIZES), n, seed=13)
+    bs = torch.tensor(SIZES)
+    out, agrad, bgrad = oracle.gmm_autograd_loop(a, b, bs, trans_b, grad)
+    torch.testing.assert_close(out, oracle.gmm_c(a, b, bs, trans_b=trans_b)[0], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(agrad, oracle.gmm_c(grad, b, bs, trans_b=not trans_b)[0], rtol=1e-5, atol=1e-5)
+    lhs, rhs = (grad, a) if trans_b else (a, grad)
+    want_bg = oracle.gmm_c(lhs, rhs, bs, trans_a=True)[0]
+    assert bgrad.shape == b.shape == want_bg.shape
+    torch.testing.assert_close(bgrad, want_bg, rtol=1e-5, atol=1e-5)
+
+
+def test_tolerance_scales_with_the_data(oracle):
+    # an all-zero answer against small expected values must fail; unit-scale data keeps atol 1e-2
+    want = torch.full((64, 64), 3e-3)
+    assert oracle.max_violation(torch.zeros(64, 64), want) > 0
+    assert oracle.max_violation(want * 1.01, want) <= 0
+    assert abs(oracle.atol_for(torch.randn(1000, 100)) - 1e-2) < 1e-3
+    assert oracle.atol_for(torch.full((8, 8), 50.0)) == 1e-2
+
+
 def test_zero_k_known_answer(oracle):
     # grouped_gemm/ops_test.py:143-158: ones x ones over k rows is exactly k
     a = torch.ones(192, 128, dtype=torch.bfloat16)
