@@ -72,9 +72,21 @@ bool use_short_shape(int64_t num_groups, int64_t tokens, int trans_a) {
   return !trans_a && num_groups > 0 && tokens < (int64_t)kShortBelow * num_groups;
 }
 
+// Scratch of gg_gmm_no_alloc: the workspace of gg_gmm (arrival counters, then partial tiles) as a
+// static array, one copy per device that loads this library, held until the process ends.  In
+// host code `scratch` is only a handle for hipGetSymbolAddress; kernels get the address that
+// call returns for the current device (DeviceInfo::scratch).
+static __device__ __align__(256) unsigned char scratch[GG_WORKSPACE_BYTES];
+
+// Most workgroups a launch may have for the static scratch to hold one partial tile each.
+constexpr int kStaticScratchGrid = (GG_WORKSPACE_BYTES - gg::kWsCounterBytes) / (256 * 256 * 4);
+
+__global__ void clear_counters_kernel(int* counters) { counters[threadIdx.x] = 0; }
+
 struct DeviceInfo {
   int cus = 0;
   bool ok = false;
+  unsigned char* scratch = nullptr;   // device address of `scratch` on this device
 };
 
 // Per device, once: the architecture check and the LDS limit of every kernel variant.
@@ -91,6 +103,9 @@ int device_info(DeviceInfo* out) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
       return fail(GG_EHIP, "this library is built for gfx950 only, device is %s", prop.gcnArchName);
     for (int i = 0; i < kNumVariants; ++i) GG_HIP(kVariantGetters[i]()->prepare());
+    void* scratch_address = nullptr;
+    GG_HIP(hipGetSymbolAddress(&scratch_address, HIP_SYMBOL(scratch)));
+    cache[dev].scratch = static_cast<unsigned char*>(scratch_address);
     cache[dev].cus = prop.multiProcessorCount;
     cache[dev].ok = true;
   }
@@ -131,7 +146,8 @@ int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens,
   return GG_OK;
 }
 
-int gmm_impl(const gg_gmm_args& g) {
+// static_scratch: use the device's static scratch array as the workspace (gg_gmm_no_alloc).
+int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   const int64_t num_groups = g.num_groups, tokens = g.tokens;
   const int64_t hidden_in = g.hidden_in, hidden_out = g.hidden_out;
   const int trans_a = g.trans_a != 0, trans_b = g.trans_b != 0;
@@ -188,7 +204,21 @@ int gmm_impl(const gg_gmm_args& g) {
                 GG_FLAG_ROW_PIECES == gg::kFlagRowPieces, "the header's flags are the kernel's");
   p.flags = g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ONE_CLASS | GG_FLAG_ROW_PIECES);
   p.sched_out = nullptr;
-  if (g.workspace != nullptr) {
+  if (static_scratch) {
+    if (g.workspace != nullptr)
+      return fail(GG_EINVAL, "gg_gmm_no_alloc brings its own scratch: workspace must be NULL");
+    if (info.cus > kStaticScratchGrid)
+      return fail(GG_ELIMIT, "the static scratch serves launches of up to %d workgroups, this device has %d "
+                  "compute units", kStaticScratchGrid, info.cus);
+    p.workspace = reinterpret_cast<char*>(info.scratch);
+    p.ws_slots = (int32_t)(((uint64_t)GG_WORKSPACE_BYTES - gg::kWsCounterBytes) / ((uint64_t)bm * bn * 4));
+    if (p.ws_slots > 1024) p.ws_slots = 1024;
+    // Every call on this device shares the array and finds what the last call left: the arrival
+    // counters must start at zero (a fill kernel, not a memset: callers may be capturing a graph).
+    hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(gg::kWsCounterBytes / 4), 0, stream,
+                       reinterpret_cast<int*>(info.scratch));
+    GG_HIP(hipGetLastError());
+  } else if (g.workspace != nullptr) {
     if (reinterpret_cast<uintptr_t>(g.workspace) & 255)
       return fail(GG_ELIMIT, "the workspace must be 256-byte aligned");
     const uint64_t slot_bytes = (uint64_t)bm * bn * 4;
@@ -268,6 +298,14 @@ int gg_gmm(const gg_gmm_args* args) {
     return fail(GG_EINVAL, "gg_gmm_args.struct_bytes is %u, this library expects %zu", args->struct_bytes,
                 sizeof(gg_gmm_args));
   return gmm_impl(*args);
+}
+
+int gg_gmm_no_alloc(const gg_gmm_args* args) {
+  if (args == nullptr) return fail(GG_EINVAL, "args is null");
+  if (args->struct_bytes != sizeof(gg_gmm_args))
+    return fail(GG_EINVAL, "gg_gmm_args.struct_bytes is %u, this library expects %zu", args->struct_bytes,
+                sizeof(gg_gmm_args));
+  return gmm_impl(*args, /*static_scratch=*/true);
 }
 
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,

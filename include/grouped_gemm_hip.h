@@ -156,6 +156,21 @@ typedef struct gg_gmm_args {
 int gg_gmm(const gg_gmm_args* args);
 
 /*
+ * gg_gmm for callers that cannot allocate and have no workspace to bring: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  Same arguments and same results as gg_gmm called with a workspace of
+ * GG_WORKSPACE_BYTES, except that args->workspace must be NULL: the partial tiles and arrival
+ * counters live in a static device array of GG_WORKSPACE_BYTES (64 MiB + 4 KiB) inside the
+ * library, one per GPU, held until the process ends.  Calls no hipMalloc, hipFree or any
+ * allocating routine; the counters are cleared by a small fill kernel on the stream ahead of the
+ * GEMM launch.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU
+ * (different streams, different threads) race on it and must be serialised by the caller.
+ * The array holds one partial tile per workgroup of a launch of up to 256 workgroups: a device
+ * with more compute units is rejected (GG_ELIMIT), as is a non-NULL workspace (GG_EINVAL).
+ */
+int gg_gmm_no_alloc(const gg_gmm_args* args);
+
+/*
  * Runs only the on-device scheduler of gg_gmm_bf16 (same device code, same
  * arguments) and writes what it derived to `table_out`, a device buffer of
  * num_groups * GG_SCHED_COLS int64: per group the problem (m, n, k), leading
