@@ -59,7 +59,8 @@ def variant_indices():
 
 
 def build_hip(force=False, jobs=None):
-    headers = [os.path.join(CSRC, f) for f in ("gmm_kernel.hpp", "gmm_variants.hpp", "gmm_variants.def")]
+    headers = [os.path.join(CSRC, f) for f in ("gmm_kernel.hpp", "gmm_generic.hpp", "gmm_variants.hpp",
+                                               "gmm_variants.def")]
     headers.append(os.path.join(ROOT, "include", "grouped_gemm_hip.h"))
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     os.makedirs(OBJ_DIR, exist_ok=True)
@@ -67,6 +68,9 @@ def build_hip(force=False, jobs=None):
     for i in variant_indices():
         units.append((os.path.join(CSRC, "gmm_variant.hip"), os.path.join(OBJ_DIR, f"gmm_variant_{i}.o"),
                       [f"-DGG_VARIANT_INDEX={i}"]))
+    for dt in range(4):   # gmm_generic.hpp, one translation unit per element type
+        units.append((os.path.join(CSRC, "gmm_generic_variant.hip"), os.path.join(OBJ_DIR, f"gmm_generic_{dt}.o"),
+                      [f"-DGG_GENERIC_DT={dt}"]))
     todo = [u for u in units if force or not _newer(u[1], [u[0]] + headers)]
     jobs = jobs or min(len(todo) or 1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1)))
     if todo:

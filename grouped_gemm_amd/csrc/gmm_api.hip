@@ -10,9 +10,14 @@
 #include <cstring>
 #include <mutex>
 
+#include "gmm_generic.hpp"
 #include "gmm_variants.hpp"
 
 namespace gg {
+const GenericOps* generic_ops_0();
+const GenericOps* generic_ops_1();
+const GenericOps* generic_ops_2();
+const GenericOps* generic_ops_3();
 #define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_) const VariantOps* variant_ops_##index();
 #include "gmm_variants.def"
 #undef GG_VARIANT
@@ -46,6 +51,18 @@ const gg::VariantOps* (*const kVariantGetters[])() = {
 #undef GG_VARIANT
 };
 constexpr int kNumVariants = sizeof(kVariantGetters) / sizeof(kVariantGetters[0]);
+
+static_assert(GG_DTYPE_BF16 == gg::kBF16 && GG_DTYPE_F16 == gg::kF16 && GG_DTYPE_F8E4M3 == gg::kF8E4M3 &&
+              GG_DTYPE_F8E5M2 == gg::kF8E5M2, "the header's element types are the kernels'");
+
+const gg::GenericOps* generic_ops(int dt) {
+  switch (dt) {
+    case gg::kBF16: return gg::generic_ops_0();
+    case gg::kF16: return gg::generic_ops_1();
+    case gg::kF8E4M3: return gg::generic_ops_2();
+    default: return gg::generic_ops_3();
+  }
+}
 
 const gg::VariantOps* find_variant(int dt, int layout, int shape, int epilogue) {
   for (int i = 0; i < kNumVariants; ++i) {
@@ -137,9 +154,6 @@ int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens,
   if (num_groups < 0 || tokens < 0 || hidden_in < 0 || hidden_out < 0)
     return fail(GG_EINVAL, "negative dimension");
   if (num_groups > 0 && batch_sizes == nullptr) return fail(GG_EINVAL, "batch_sizes is null");
-  if (hidden_in % 8 != 0 || hidden_out % 8 != 0)
-    return fail(GG_ELIMIT, "hidden_in (%lld) and hidden_out (%lld) must be multiples of 8",
-                (long long)hidden_in, (long long)hidden_out);
   if (hidden_in >= (1 << 22) || hidden_out >= (1 << 22))
     return fail(GG_ELIMIT, "hidden sizes must be below 2^22");
   if (tokens >= (int64_t(1) << 31)) return fail(GG_ELIMIT, "tokens must be below 2^31");
@@ -154,8 +168,13 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   const bool out_f32 = g.accumulate_f32 != 0;
   int rc = check_common(g.batch_sizes, num_groups, tokens, hidden_in, hidden_out, trans_a, trans_b);
   if (rc != GG_OK) return rc;
-  if (g.dtype != GG_DTYPE_BF16 && g.dtype != GG_DTYPE_F16)
-    return fail(GG_EINVAL, "dtype must be GG_DTYPE_BF16 or GG_DTYPE_F16");
+  if (g.dtype < GG_DTYPE_BF16 || g.dtype > GG_DTYPE_F8E5M2)
+    return fail(GG_EINVAL, "dtype must be one of GG_DTYPE_*");
+  const int elem_bytes = g.dtype == GG_DTYPE_F8E4M3 || g.dtype == GG_DTYPE_F8E5M2 ? 1 : 2;
+  if (trans_a && g.c_row_index != nullptr)
+    return fail(GG_EINVAL, "c_row_index scatters output rows; the trans_a output has none per token");
+  if (!trans_a && g.b_row_index != nullptr)
+    return fail(GG_EINVAL, "b_row_index gathers rows of b; only the trans_a layout has a row per token in b");
   if (out_f32 && !trans_a)
     return fail(GG_EINVAL, "the fp32-accumulated output exists for the trans_a layout only");
   if (out_f32 && (hidden_in >= (1 << 20) || hidden_out >= (1 << 20)))
@@ -165,9 +184,20 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   if (hidden_out == 0 || (trans_a ? hidden_in == 0 : tokens == 0)) return GG_OK;
   if (g.c == nullptr) return fail(GG_EINVAL, "c is null");
   if (tokens > 0 && (g.a == nullptr || g.b == nullptr)) return fail(GG_EINVAL, "a or b is null");
-  // rows are fetched and stored 16 bytes at a time
-  if ((reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b) | reinterpret_cast<uintptr_t>(g.c)) & 15)
-    return fail(GG_ELIMIT, "a, b and c must be 16-byte aligned");
+  const uintptr_t address_bits =
+      reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b) | reinterpret_cast<uintptr_t>(g.c);
+  if (address_bits & (uintptr_t)(elem_bytes - 1) || reinterpret_cast<uintptr_t>(g.c) & (out_f32 ? 3 : 1))
+    return fail(GG_ELIMIT, "a, b and c must be aligned to their element size");
+  // The streaming kernels fetch and store rows 16 bytes at a time: two-byte elements, hidden sizes
+  // that are multiples of 8, operands on 16-byte boundaries, rows in place.  Everything else goes
+  // to the kernels of gmm_generic.hpp, VEC elements at a time.
+  const bool generic = elem_bytes != 2 || hidden_in % 8 != 0 || hidden_out % 8 != 0 || (address_bits & 15) ||
+                       g.a_row_index != nullptr || g.b_row_index != nullptr || g.c_row_index != nullptr;
+  int vec = 8;
+  if (generic) {
+    while (vec > 1 && (hidden_in % vec != 0 || hidden_out % vec != 0 || (address_bits & (uintptr_t)(vec * 2 - 1))))
+      vec >>= 1;
+  }
 
   // Host-resident sizes are validated here; they travel in the kernel argument block.
   if (!g.batch_sizes_on_device) {
@@ -185,12 +215,15 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   if (rc != GG_OK) return rc;
   hipStream_t stream = static_cast<hipStream_t>(g.stream);
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
-  const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
-  const int bm = short_shape ? Short::BM : Wide::BM, bn = short_shape ? Short::BN : Wide::BN;
-  const gg::VariantOps* variant = find_variant(g.dtype == GG_DTYPE_F16 ? gg::kF16 : gg::kBF16, layout,
-                                               short_shape ? Short::kId : Wide::kId,
-                                               out_f32 ? gg::kEpiAccF32 : gg::kEpiStore);
-  if (variant == nullptr) return fail(GG_EINVAL, "no kernel for this combination of arguments");
+  const bool short_shape = !generic && use_short_shape(num_groups, tokens, trans_a);
+  const int bm = generic ? gg::kGenericTileM : (short_shape ? Short::BM : Wide::BM);
+  const int bn = generic ? gg::kGenericTileN : (short_shape ? Short::BN : Wide::BN);
+  const gg::VariantOps* variant = nullptr;
+  if (!generic) {
+    variant = find_variant(g.dtype, layout, short_shape ? Short::kId : Wide::kId,
+                           out_f32 ? gg::kEpiAccF32 : gg::kEpiStore);
+    if (variant == nullptr) return fail(GG_EINVAL, "no kernel for this combination of arguments");
+  }
 
   gg::GmmParams p{};
   p.a = static_cast<const char*>(g.a);
@@ -218,7 +251,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(gg::kWsCounterBytes / 4), 0, stream,
                        reinterpret_cast<int*>(info.scratch));
     GG_HIP(hipGetLastError());
-  } else if (g.workspace != nullptr) {
+  } else if (g.workspace != nullptr && !generic) {
     if (reinterpret_cast<uintptr_t>(g.workspace) & 255)
       return fail(GG_ELIMIT, "the workspace must be 256-byte aligned");
     const uint64_t slot_bytes = (uint64_t)bm * bn * 4;
@@ -264,7 +297,20 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     if (tiles == 0) continue;
     // the full grid also for few tiles: the last round's tiles may be cut into pieces for
     // the workgroups that would otherwise idle
-    GG_HIP(variant->launch(p, hs, info.cus, stream));
+    if (generic) {
+      gg::GenericParams gp;
+      gp.p = p;
+      gp.p.workspace = nullptr;
+      gp.p.ws_slots = 0;
+      gp.a_rows = g.a_row_index;
+      gp.b_rows = g.b_row_index;
+      gp.c_rows = g.c_row_index;
+      // light workgroups (28 KiB of LDS): two per compute unit
+      const int64_t grid = tiles < 2 * info.cus ? tiles : 2 * info.cus;
+      GG_HIP(generic_ops(g.dtype)->launch(layout, vec, out_f32, gp, hs, (int)grid, stream));
+    } else {
+      GG_HIP(variant->launch(p, hs, info.cus, stream));
+    }
   }
   return GG_OK;
 }

@@ -35,4 +35,14 @@ struct VariantOps {
   hipError_t (*launch)(const GmmParams& p, const HostSizes& hs, int grid, hipStream_t stream);
 };
 
+// The kernels of gmm_generic.hpp for one element type (gmm_generic_variant.hip).
+struct GenericParams;
+struct GenericOps {
+  int dt;
+  hipError_t (*launch)(int layout, int vec, bool acc_f32, const GenericParams& gp, const HostSizes& hs,
+                       int grid, hipStream_t stream);
+};
+constexpr int kGenericTileM = 128, kGenericTileN = 128;
+constexpr int kNumElementTypes = 4;   // bf16, f16, f8 e4m3, f8 e5m2
+
 }  // namespace gg

@@ -20,10 +20,33 @@ namespace grouped_gemm {
 
 namespace {
 
+bool IsFloat8(torch::ScalarType t) { return t == torch::kFloat8_e4m3fn || t == torch::kFloat8_e5m2; }
+
+// Element type of c for operands of type `t`: the same for the two-byte types, bf16 for fp8.
+torch::ScalarType OutputType(torch::ScalarType t) { return IsFloat8(t) ? torch::kBFloat16 : t; }
+
+int DtypeCode(torch::ScalarType t) {
+  switch (t) {
+    case torch::kFloat16: return GG_DTYPE_F16;
+    case torch::kFloat8_e4m3fn: return GG_DTYPE_F8E4M3;
+    case torch::kFloat8_e5m2: return GG_DTYPE_F8E5M2;
+    default: return GG_DTYPE_BF16;
+  }
+}
+
+// Row indices of the fused gather / scatter forms (see gg_gmm): undefined tensors mean "rows in place".
+struct RowIndices {
+  torch::Tensor a, b, c;
+  bool any() const { return a.defined() || b.defined() || c.defined(); }
+};
+
 // `on_device` false skips the checks that a tensor lives on the GPU, so that the shape,
 // rank and dtype rules can be exercised with CPU tensors on a machine without one.
+// With row indices, `tokens` (the rows of the product) is the length of the index instead of the
+// row count of the tensor it redirects.
 void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
-              const torch::Tensor& batch_sizes, bool trans_a, bool trans_b, bool on_device) {
+              const torch::Tensor& batch_sizes, bool trans_a, bool trans_b, bool on_device,
+              const RowIndices& rows = RowIndices()) {
   // Only one of the operands may be transposed (csrc/grouped_gemm.cu:476).
   TORCH_CHECK(!(trans_a && trans_b), "grouped_gemm: trans_a and trans_b cannot both be set");
 
@@ -37,8 +60,8 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
   // as well, for all three tensors alike; the reference takes bfloat16 only.
   if (on_device) TORCH_CHECK(a.is_cuda(), "grouped_gemm: a must be a GPU tensor");
   TORCH_CHECK(a.ndimension() == 2, "grouped_gemm: a must be 2-d");
-  TORCH_CHECK(a.scalar_type() == torch::kBFloat16 || a.scalar_type() == torch::kFloat16,
-              "grouped_gemm: a must be bfloat16 (or float16)");
+  TORCH_CHECK(a.scalar_type() == torch::kBFloat16 || a.scalar_type() == torch::kFloat16 || IsFloat8(a.scalar_type()),
+              "grouped_gemm: a must be bfloat16 (or float16, float8_e4m3fn, float8_e5m2)");
 
   // b, c: bf16 on the GPU (csrc/grouped_gemm.cu:503-506).
   if (on_device) {
@@ -46,14 +69,25 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
     TORCH_CHECK(c.is_cuda(), "grouped_gemm: c must be a GPU tensor");
   }
   TORCH_CHECK(b.scalar_type() == a.scalar_type(), "grouped_gemm: b must be bfloat16 (the element type of a)");
-  TORCH_CHECK(c.scalar_type() == a.scalar_type(), "grouped_gemm: c must be bfloat16 (the element type of a)");
+  TORCH_CHECK(c.scalar_type() == OutputType(a.scalar_type()),
+              "grouped_gemm: c must be bfloat16 (the element type of a; bfloat16 for float8 operands)");
+  for (const torch::Tensor* idx : {&rows.a, &rows.b, &rows.c}) {
+    if (!idx->defined()) continue;
+    TORCH_CHECK(idx->ndimension() == 1 && idx->scalar_type() == torch::kInt32 && idx->is_contiguous(),
+                "grouped_gemm: a row index must be a contiguous 1-d int32 tensor");
+    if (on_device) TORCH_CHECK(idx->is_cuda() && idx->device() == a.device(), "grouped_gemm: a row index must be on a's GPU");
+  }
+  TORCH_CHECK(!(trans_a && rows.c.defined()), "grouped_gemm: the trans_a output has no row per token to scatter");
+  TORCH_CHECK(trans_a || !rows.b.defined(), "grouped_gemm: only the trans_a layout has a row per token in b");
+  const int64_t tokens = rows.a.defined() ? rows.a.size(0) : a.size(0);
 
   if (trans_a) {
     // b (tokens, hidden_out), c (num_experts, hidden_in, hidden_out)
     // (csrc/grouped_gemm.cu:513-522).
     TORCH_CHECK(b.ndimension() == 2, "grouped_gemm: with trans_a, b must be 2-d");
     TORCH_CHECK(c.ndimension() == 3, "grouped_gemm: with trans_a, c must be 3-d");
-    TORCH_CHECK(b.size(0) == a.size(0), "grouped_gemm: a and b must have the same number of rows");
+    TORCH_CHECK((rows.b.defined() ? rows.b.size(0) : b.size(0)) == tokens,
+                "grouped_gemm: a and b must have the same number of rows");
     TORCH_CHECK(c.size(0) == batch_sizes.size(0), "grouped_gemm: c.size(0) must equal the number of experts");
     TORCH_CHECK(c.size(1) == a.size(1), "grouped_gemm: c.size(1) must equal a.size(1)");
     TORCH_CHECK(c.size(2) == b.size(1), "grouped_gemm: c.size(2) must equal b.size(1)");
@@ -68,8 +102,13 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
     // The reference leaves the shape of c unchecked here; a wrong one would make the
     // kernel write outside c, so it is rejected.
     const int64_t hidden_out = trans_b ? b.size(1) : b.size(2);
-    TORCH_CHECK(c.size(0) == a.size(0) && c.size(1) == hidden_out,
-                "grouped_gemm: c must have shape (tokens, hidden_out)");
+    if (rows.c.defined()) {
+      TORCH_CHECK(rows.c.size(0) == tokens, "grouped_gemm: c_rows needs one entry per row of the product");
+      TORCH_CHECK(c.size(1) == hidden_out, "grouped_gemm: c must have hidden_out columns");
+    } else {
+      TORCH_CHECK(c.size(0) == tokens && c.size(1) == hidden_out,
+                  "grouped_gemm: c must have shape (tokens, hidden_out)");
+    }
   }
 
   // Transposition goes through the flags only (csrc/grouped_gemm.cu:538-540).
@@ -107,7 +146,7 @@ torch::Tensor Workspace(const torch::Device& device, hipStream_t stream) {
 }
 
 void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c, const torch::Tensor& batch_sizes,
-         bool trans_a, bool trans_b, bool accumulate_f32, int64_t flags) {
+         bool trans_a, bool trans_b, bool accumulate_f32, int64_t flags, const RowIndices& rows = RowIndices()) {
   torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
   c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
@@ -115,7 +154,7 @@ void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
   torch::Tensor ws = Workspace(a.device(), stream);
   gg_gmm_args g = {};
   g.struct_bytes = sizeof(g);
-  g.dtype = a.scalar_type() == torch::kFloat16 ? GG_DTYPE_F16 : GG_DTYPE_BF16;
+  g.dtype = DtypeCode(a.scalar_type());
   g.a = a.data_ptr();
   g.b = b.data_ptr();
   g.c = c.data_ptr();
@@ -125,7 +164,10 @@ void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
   g.trans_b = trans_b ? 1 : 0;
   g.accumulate_f32 = accumulate_f32 ? 1 : 0;
   g.num_groups = sizes.size(0);
-  g.tokens = a.size(0);
+  g.tokens = rows.a.defined() ? rows.a.size(0) : a.size(0);
+  g.a_row_index = rows.a.defined() ? rows.a.data_ptr<int32_t>() : nullptr;
+  g.b_row_index = rows.b.defined() ? rows.b.data_ptr<int32_t>() : nullptr;
+  g.c_row_index = rows.c.defined() ? rows.c.data_ptr<int32_t>() : nullptr;
   g.hidden_in = a.size(1);
   g.hidden_out = trans_a ? b.size(1) : (trans_b ? b.size(1) : b.size(2));
   g.workspace = ws.data_ptr();
@@ -149,6 +191,19 @@ void GroupedGemmWithFlags(torch::Tensor a, torch::Tensor b, torch::Tensor c, tor
                           bool trans_a, bool trans_b, int64_t flags) {
   Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/true);
   Run(a, b, c, batch_sizes, trans_a, trans_b, /*accumulate_f32=*/false, flags);
+}
+
+// gmm with row indices: a gather fused into the loads of a (and of b with trans_a), a scatter
+// fused into the stores of c.  An undefined (None) index leaves those rows in place.
+void GroupedGemmIndexed(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes,
+                        bool trans_a, bool trans_b, c10::optional<torch::Tensor> a_rows,
+                        c10::optional<torch::Tensor> b_rows, c10::optional<torch::Tensor> c_rows) {
+  RowIndices rows;
+  if (a_rows.has_value()) rows.a = *a_rows;
+  if (b_rows.has_value()) rows.b = *b_rows;
+  if (c_rows.has_value()) rows.c = *c_rows;
+  Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/true, rows);
+  Run(a, b, c, batch_sizes, trans_a, trans_b, /*accumulate_f32=*/false, /*flags=*/0, rows);
 }
 
 // c (num_experts, hidden_in, hidden_out) fp32 += per expert a_e^T @ b_e; see gg_gmm_bf16_acc_f32.
@@ -191,6 +246,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         [](torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes, bool trans_a,
            bool trans_b) { Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/false); },
         "Shape, rank and dtype checks of gmm without the device checks.");
+  m.def("gmm_indexed", &GroupedGemmIndexed, "gmm with fused row gather / scatter.", py::arg("a"), py::arg("b"),
+        py::arg("c"), py::arg("batch_sizes"), py::arg("trans_a"), py::arg("trans_b"), py::arg("a_rows") = py::none(),
+        py::arg("b_rows") = py::none(), py::arg("c_rows") = py::none());
   m.def("gmm_with_flags", &GroupedGemmWithFlags, "gmm with GG_FLAG_* bits (testing).");
   m.attr("flag_whole_tiles") = GG_FLAG_WHOLE_TILES;
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,

@@ -39,6 +39,81 @@ def gmm(a, b, batch_sizes, trans_b=False):
     return GroupedGemm.apply(a, b, batch_sizes, trans_b)
 
 
+# --------------------------------------------------- fused permutation (gather / scatter)
+#
+# MoE layers sort their tokens by expert before the first grouped GEMM and put the rows back after
+# the last one.  The reference's operator takes rows already sorted (ops.py:8); these two forms
+# take the permutation as an index and do the move inside the GEMM's loads or stores, which saves
+# a full pass over the activations each.  Not part of the reference's surface.
+
+class GroupedGemmGather(torch.autograd.Function):
+    """out[r] = x[row_index[r]] @ w[expert of r]: rows are gathered while they are loaded.  An
+    index may name a row of x several times (top-k routing)."""
+
+    @staticmethod
+    def forward(ctx, x, w, batch_sizes, row_index, trans_b):
+        ctx.save_for_backward(x, w, batch_sizes, row_index)
+        ctx.trans_b = trans_b
+        return backend.gmm_indexed(x, w, batch_sizes, trans_b=trans_b, a_rows=row_index)
+
+    @staticmethod
+    def backward(ctx, grad):
+        grad = grad.contiguous()
+        x, w, batch_sizes, row_index = ctx.saved_tensors
+        xgrad = wgrad = None
+        if ctx.needs_input_grad[0]:
+            # rows of x that several sorted rows came from collect several gradients: a sum, not
+            # a store, so it is not fused
+            sorted_grad = backend.gmm(grad, w, batch_sizes, trans_b=not ctx.trans_b)
+            xgrad = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            xgrad.index_add_(0, row_index.long(), sorted_grad.float())
+            xgrad = xgrad.to(x.dtype)
+        if ctx.needs_input_grad[1]:
+            if ctx.trans_b:
+                wgrad = backend.gmm_indexed(grad, x, batch_sizes, trans_a=True, b_rows=row_index)
+            else:
+                wgrad = backend.gmm_indexed(x, grad, batch_sizes, trans_a=True, a_rows=row_index)
+        return xgrad, wgrad, None, None, None
+
+
+class GroupedGemmScatter(torch.autograd.Function):
+    """out[row_index[r]] = a[r] @ w[expert of r] for a permutation row_index of 0..rows-1: rows are
+    put back in their original order while they are stored."""
+
+    @staticmethod
+    def forward(ctx, a, w, batch_sizes, row_index, trans_b):
+        ctx.save_for_backward(a, w, batch_sizes, row_index)
+        ctx.trans_b = trans_b
+        hidden_out = w.shape[1] if trans_b else w.shape[2]
+        out = torch.empty(a.shape[0], hidden_out, dtype=a.dtype, device=a.device)
+        return backend.gmm_indexed(a, w, batch_sizes, trans_b=trans_b, c=out, c_rows=row_index)
+
+    @staticmethod
+    def backward(ctx, grad):
+        grad = grad.contiguous()
+        a, w, batch_sizes, row_index = ctx.saved_tensors
+        agrad = wgrad = None
+        if ctx.needs_input_grad[0]:
+            agrad = backend.gmm_indexed(grad, w, batch_sizes, trans_b=not ctx.trans_b, a_rows=row_index)
+        if ctx.needs_input_grad[1]:
+            if ctx.trans_b:
+                wgrad = backend.gmm_indexed(grad, a, batch_sizes, trans_a=True, a_rows=row_index)
+            else:
+                wgrad = backend.gmm_indexed(a, grad, batch_sizes, trans_a=True, b_rows=row_index)
+        return agrad, wgrad, None, None, None
+
+
+def gmm_gather(x, w, batch_sizes, row_index, trans_b=False):
+    """gmm(x[row_index], w, batch_sizes, trans_b) with the gather fused into the GEMM."""
+    return GroupedGemmGather.apply(x, w, batch_sizes, row_index, trans_b)
+
+
+def gmm_scatter(a, w, batch_sizes, row_index, trans_b=False):
+    """out with out[row_index] = gmm(a, w, batch_sizes, trans_b): the scatter fused into the GEMM.
+    row_index must be a permutation of the rows."""
+    return GroupedGemmScatter.apply(a, w, batch_sizes, row_index, trans_b)
+
+
 # ------------------------------------------------------------------ traceable form
 #
 # The same operator registered with torch.library, so that torch.compile sees one opaque node

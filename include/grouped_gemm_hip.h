@@ -40,6 +40,8 @@ extern "C" {
 /* Element types of a and b (and of c, unless it is the fp32 accumulator). */
 #define GG_DTYPE_BF16 0
 #define GG_DTYPE_F16 1
+#define GG_DTYPE_F8E4M3 2   /* OCP e4m3 (torch.float8_e4m3fn) in a and b, bf16 in c */
+#define GG_DTYPE_F8E5M2 3   /* OCP e5m2 (torch.float8_e5m2) in a and b, bf16 in c */
 
 /* Bytes of workspace that let any call cut the tiles of its last, partly filled round along the
  * depth (see gg_gmm): 4096 bytes of arrival counters and 256 partial tiles of 256 x 256 floats. */
@@ -85,9 +87,10 @@ int gg_init(void);
  * One persistent launch (one per 512 groups).  Uses no workspace: the tiles of a partly filled
  * last round are cut along their rows only; gg_gmm with a workspace cuts them along the depth.
  *
- * Limits (GG_ELIMIT): a, b and c 16-byte aligned, hidden_in and hidden_out multiples of 8
- * (16-byte rows, the same alignment the reference's kernel configuration assumes,
- * csrc/grouped_gemm.cu:41-66) and below 2^22; tokens below 2^31.
+ * Limits (GG_ELIMIT): hidden_in and hidden_out below 2^22; tokens below 2^31.  Hidden sizes that
+ * are multiples of 8 with a, b and c on 16-byte boundaries (the alignment the reference's kernel
+ * configuration assumes, csrc/grouped_gemm.cu:41-66) run on the streaming kernels, other sizes and
+ * alignments on slower, general ones (see gg_gmm).
  */
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,
                 int batch_sizes_on_device, int64_t num_groups, int64_t tokens,
@@ -115,8 +118,23 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  * what the reference's entry point (csrc/grouped_gemm.cu:470-564) has no argument for.  Zero
  * the struct, set struct_bytes = sizeof(gg_gmm_args), fill in what is needed.
  *
- *   dtype         GG_DTYPE_BF16 or GG_DTYPE_F16: element type of a, b and c (the reference
- *                 rejects everything but bf16, csrc/grouped_gemm.cu:492, 505-506).
+ *   dtype         GG_DTYPE_*: element type of a and b, and of c for the two-byte types (fp8
+ *                 operands give a bf16 c).  The reference rejects everything but bf16
+ *                 (csrc/grouped_gemm.cu:492, 505-506).
+ *   hidden_in, hidden_out
+ *                 Any size below 2^22 (the reference's default build runs any size through
+ *                 cuBLAS, csrc/grouped_gemm.cu:373-394, its grouped kernel assumes multiples of
+ *                 8, :469).  Multiples of 8 with 16-byte aligned two-byte operands run on the
+ *                 streaming kernels; everything else on slower, general ones.
+ *   a_row_index   int32[tokens] on the device, or NULL: row r of the product's left operand is
+ *                 row a_row_index[r] of `a` (a gather fused into the load: `a` is the tensor
+ *                 before the permutation that sorts rows by group, and may have any number of
+ *                 rows).  The reference takes rows already sorted (grouped_gemm/ops.py:8).
+ *   b_row_index   the same for the rows of b, trans_a layout only.
+ *   c_row_index   int32[tokens] on the device, or NULL: row r of the output is stored to row
+ *                 c_row_index[r] of c (a scatter fused into the store; not with trans_a).  Rows of
+ *                 c that no index names are not touched.  Indices are not checked: each must
+ *                 name a row that exists, and c_row_index must not name a row twice.
  *   accumulate_f32  1: c is fp32 and is added to (trans_a = 1 only), as gg_gmm_bf16_acc_f32.
  *   workspace, workspace_bytes
  *                 Device memory the call may use for partial results, or NULL.  When the last
@@ -151,6 +169,9 @@ typedef struct gg_gmm_args {
   int32_t flags;
   int32_t reserved0;
   void* stream;
+  const int32_t* a_row_index;
+  const int32_t* b_row_index;
+  const int32_t* c_row_index;
 } gg_gmm_args;
 
 int gg_gmm(const gg_gmm_args* args);

@@ -541,7 +541,8 @@ class GmmArgs(ctypes.Structure):
                 ("num_groups", ctypes.c_int64), ("tokens", ctypes.c_int64),
                 ("hidden_in", ctypes.c_int64), ("hidden_out", ctypes.c_int64),
                 ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_uint64),
-                ("flags", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("stream", ctypes.c_void_p)]
+                ("flags", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("stream", ctypes.c_void_p),
+                ("a_row_index", ctypes.c_void_p), ("b_row_index", ctypes.c_void_p), ("c_row_index", ctypes.c_void_p)]
 
 
 def _gmm_args(lib, a, b, c, sizes, on_device, tokens, hin, hout, trans_a, trans_b, flags=0, workspace=None,
@@ -793,6 +794,216 @@ def test_float16_autograd_and_mixed_dtypes(ops, oracle, trans_b):
     assert float((c.double().cpu() - want_c).abs().max()) <= 1e-4 * float(want_c.abs().max())
 
 
+# ------------------------------------- any hidden size, any alignment (the general kernels)
+
+def _odd_cases(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    pool = [1, 2, 3, 5, 7, 12, 20, 33, 100, 130, 250, 1001]
+    cases = []
+    for _ in range(n):
+        e = r(1, 6)
+        sizes = [r(0, 3) * 64 + r(-3, 70) for _ in range(e)]
+        sizes = [max(0, x) for x in sizes]
+        cases.append((sizes, pool[r(0, len(pool) - 1)], pool[r(0, len(pool) - 1)]))
+    cases += [([130, 0, 7], 12, 100), ([300], 1001, 1001), ([5, 129], 100, 12), ([64, 64], 1, 1)]
+    return cases
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_hidden_sizes_that_are_not_multiples_of_8(ops, oracle, layout, dtype):
+    # the reference's default build takes any hidden size (csrc/grouped_gemm.cu:373-394); sizes
+    # that are multiples of 4, of 2, and odd ones, each through its own vector width
+    trans_a, trans_b = layout
+    for idx, (sizes, hin, hout) in enumerate(_odd_cases(10, seed=51 + int(trans_a) + 2 * int(trans_b))):
+        _announce("any size", layout, dtype, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(dtype)
+        else:
+            b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(dtype)
+        dev_bs = bs.cuda() if idx % 2 else bs
+        out = ops.backend.gmm(a.cuda(), b.cuda(), dev_bs, trans_a=trans_a, trans_b=trans_b)
+        want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
+        check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
+
+
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_operands_off_the_16_byte_boundary(ops, oracle, layout):
+    # views that start one, two or four elements into a buffer: same results as the aligned call
+    trans_a, trans_b = layout
+    g = torch.Generator().manual_seed(61)
+    sizes = torch.tensor([70, 0, 300, 41])
+    t, hin, hout = int(sizes.sum()), 136, 264
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+    b = torch.randn(t, hout, generator=g).to(torch.bfloat16) if trans_a else \
+        torch.randn(4, *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+    want = oracle.gmm_loop(a, b, sizes, trans_a=trans_a, trans_b=trans_b)
+
+    def shifted(x, by):
+        buf = torch.empty(x.numel() + by, dtype=x.dtype, device="cuda")
+        view = buf[by:].view(x.shape)
+        view.copy_(x)
+        assert view.data_ptr() % 16 == (2 * by) % 16
+        return view
+
+    for by_a, by_b, by_c in [(1, 0, 0), (0, 2, 0), (0, 0, 4), (1, 3, 5)]:
+        _announce("off boundary", layout, by_a, by_b, by_c)
+        c = shifted(torch.zeros(want.shape, dtype=torch.bfloat16), by_c)
+        ops.backend.gmm(shifted(a, by_a), shifted(b, by_b), sizes.cuda(), trans_a=trans_a, trans_b=trans_b, c=c)
+        check(c, want, f"shifted by {by_a}, {by_b}, {by_c} elements")
+
+
+def test_accumulated_weight_gradient_any_size(ops, oracle):
+    g = torch.Generator().manual_seed(63)
+    sizes = torch.tensor([300, 0, 17, 129])
+    t = int(sizes.sum())
+    for hin, hout in [(100, 12), (33, 1001), (7, 7)]:
+        a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+        b = torch.randn(t, hout, generator=g).to(torch.bfloat16)
+        c0 = torch.randn(4, hin, hout, generator=g)
+        c = c0.clone().cuda()
+        ops.backend.accumulate_weight_gradient(a.cuda(), b.cuda(), sizes.cuda(), c)
+        want = oracle.accumulate_weight_gradient_loop(a, b, sizes, c0)
+        assert float((c.double().cpu() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+        assert torch.equal(c[1].cpu(), c0[1])
+
+
+# ----------------------------------------------------------------------- fp8 operands
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_float8_operands(ops, oracle, layout, dtype):
+    # fp8 in a and b (OCP formats), fp32 accumulation of the exact products, one bf16 rounding on
+    # store; the oracle is the per-expert loop on the fp32 decode of the same bytes
+    trans_a, trans_b = layout
+    cases = _random_cases(6, seed=71 + int(trans_a) + 2 * int(trans_b)) + [([130, 0, 7], 100, 12), ([300], 1001, 33)]
+    for idx, (sizes, hin, hout) in enumerate(cases):
+        _announce("fp8", layout, dtype, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(dtype)
+        else:
+            b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(dtype)
+        out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda() if idx % 2 else bs, trans_a=trans_a, trans_b=trans_b)
+        assert out.dtype == torch.bfloat16
+        want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
+        check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
+
+
+# ------------------------------------------------------------- fused gather / scatter
+
+def _routing(tokens, experts, top_k, seed):
+    """Top-k routing of `tokens` rows: the sorted order (row_index[r] = source row of sorted row r),
+    the group sizes, and the position of each (token, k) pair in the sorted order."""
+    g = torch.Generator().manual_seed(seed)
+    expert = torch.stack([torch.randperm(experts, generator=g)[:top_k] for _ in range(tokens)])   # (tokens, k)
+    flat = expert.flatten()
+    order = torch.argsort(flat, stable=True)
+    sizes = torch.bincount(flat, minlength=experts).to(torch.int64)
+    return (order // top_k).to(torch.int32), sizes, order.to(torch.int32)
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+@pytest.mark.parametrize("hidden", [(136, 264), (100, 12)])
+def test_gather_and_scatter_against_indexed_oracle(ops, oracle, trans_b, hidden):
+    # gmm_indexed(a, ..., a_rows=idx) == gmm(a[idx], ...) and c[c_rows] = gmm(...), the oracle being
+    # the index applied by torch and then the pinned per-expert loop
+    hin, hout = hidden
+    row_index, sizes, order = _routing(400, 6, 2, seed=81)
+    g = torch.Generator().manual_seed(82)
+    x = torch.randn(400, hin, generator=g).to(torch.bfloat16)
+    w = torch.randn(6, *((hout, hin) if trans_b else (hin, hout)), generator=g).to(torch.bfloat16)
+    _announce("gather", trans_b, hidden)
+    got = ops.backend.gmm_indexed(x.cuda(), w.cuda(), sizes.cuda(), trans_b=trans_b, a_rows=row_index.cuda())
+    want = oracle.gmm_loop(x[row_index.long()], w, sizes, trans_b=trans_b)
+    check(got, want, "gathered rows")
+    # scatter: the sorted product goes back to (token, k) order; rows no index names stay as they were
+    a_sorted = x[row_index.long()].contiguous()
+    c = torch.full((800 + 3, hout), 7.0, dtype=torch.bfloat16, device="cuda")
+    ops.backend.gmm_indexed(a_sorted.cuda(), w.cuda(), sizes, trans_b=trans_b, c=c, c_rows=order.cuda())
+    want_c = torch.full((803, hout), 7.0)
+    want_c[order.long()] = want
+    check(c, want_c, "scattered rows")
+    assert (c[800:] == 7.0).all()
+    # both at once
+    c2 = torch.zeros(800, hout, dtype=torch.bfloat16, device="cuda")
+    ops.backend.gmm_indexed(x.cuda(), w.cuda(), sizes.cuda(), trans_b=trans_b, c=c2, a_rows=row_index.cuda(),
+                            c_rows=order.cuda())
+    check(c2, want_c[:800], "gathered and scattered")
+
+
+@pytest.mark.parametrize("hidden", [(136, 264), (33, 20)])
+def test_weight_gradient_with_gathered_rows(ops, oracle, hidden):
+    hin, hout = hidden
+    row_index, sizes, order = _routing(300, 5, 2, seed=83)
+    g = torch.Generator().manual_seed(84)
+    x = torch.randn(300, hin, generator=g).to(torch.bfloat16)
+    grad_sorted = torch.randn(600, hout, generator=g).to(torch.bfloat16)
+    _announce("gathered weight gradient", hidden)
+    got = ops.backend.gmm_indexed(x.cuda(), grad_sorted.cuda(), sizes.cuda(), trans_a=True, a_rows=row_index.cuda())
+    want = oracle.gmm_loop(x[row_index.long()], grad_sorted, sizes, trans_a=True)
+    check(got, want, "a rows gathered")
+    # b gathered: the gradient in (token, k) order, the activations sorted
+    grad_unsorted = torch.zeros_like(grad_sorted)
+    grad_unsorted[order.long()] = grad_sorted
+    a_sorted = x[row_index.long()].contiguous()
+    got = ops.backend.gmm_indexed(a_sorted.cuda(), grad_unsorted.cuda(), sizes, trans_a=True, b_rows=order.cuda())
+    check(got, want, "b rows gathered")
+
+
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_fused_permutation_autograd(ops, oracle, trans_b):
+    # a whole expert layer: gather-fused first GEMM, scatter-fused second GEMM, against the same
+    # layer written with index operations and the oracle's loops, forward and all gradients
+    hin, hmid = 136, 264
+    row_index, sizes, order = _routing(256, 4, 2, seed=85)
+    g = torch.Generator().manual_seed(86)
+    x0 = torch.randn(256, hin, generator=g).to(torch.bfloat16)
+    w1_0 = (torch.randn(4, *((hmid, hin) if trans_b else (hin, hmid)), generator=g) * 0.1).to(torch.bfloat16)
+    w2_0 = (torch.randn(4, *((hin, hmid) if trans_b else (hmid, hin)), generator=g) * 0.1).to(torch.bfloat16)
+    gout = torch.randn(512, hin, generator=g).to(torch.bfloat16)
+    x, w1, w2 = (t.cuda().requires_grad_(True) for t in (x0, w1_0, w2_0))
+    _announce("fused layer", trans_b)
+    h = ops.gmm_gather(x, w1, sizes.cuda(), row_index.cuda(), trans_b)
+    y = ops.gmm_scatter(h, w2, sizes.cuda(), order.cuda(), trans_b)       # (token, k) order
+    y.backward(gout.cuda())
+    # Reference: the same layer from index operations and the oracle's loop, stage by stage, with a
+    # bf16 rounding wherever the fused path stores a bf16 tensor (h, its gradient, the sorted
+    # input gradient), so that only fp32 summation order separates the two.
+    bf = lambda t: t.to(torch.bfloat16)
+    idx, ordr = row_index.long(), order.long()
+    h_ref = oracle.gmm_loop(x0[idx], w1_0, sizes, trans_b=trans_b)
+    y_sorted = oracle.gmm_loop(bf(h_ref), w2_0, sizes, trans_b=trans_b)
+    y_ref = torch.zeros(512, hin).index_put((ordr,), y_sorted)
+    dy_sorted = gout[ordr]
+    lhs, rhs = (dy_sorted, bf(h_ref)) if trans_b else (bf(h_ref), dy_sorted)
+    w2g_ref = oracle.gmm_loop(lhs, rhs, sizes, trans_a=True)
+    dh = bf(oracle.gmm_loop(dy_sorted, w2_0, sizes, trans_b=not trans_b))
+    lhs, rhs = (dh, x0[idx]) if trans_b else (x0[idx], dh)
+    w1g_ref = oracle.gmm_loop(lhs, rhs, sizes, trans_a=True)
+    dx_sorted = bf(oracle.gmm_loop(dh, w1_0, sizes, trans_b=not trans_b))
+    xg_ref = torch.zeros(256, hin).index_add_(0, idx, dx_sorted.float())
+
+    # outputs well above unit scale are compared in units of their root-mean-square
+    def check_scaled(got, want, what):
+        scale = max(1.0, float(want.double().pow(2).mean().sqrt()))
+        check(got.float().cpu() / scale, want / scale, what)
+
+    check_scaled(h.detach(), h_ref, "first GEMM")
+    check_scaled(y.detach(), y_ref, "second GEMM")
+    check_scaled(w2.grad, w2g_ref, "w2 gradient")
+    check_scaled(w1.grad, w1g_ref, "w1 gradient")
+    check_scaled(x.grad, xg_ref, "x gradient")
+
+
 # ------------------------------------------------- fp32-accumulated weight gradient
 
 @pytest.mark.parametrize("on_device", [False, True])
@@ -957,8 +1168,6 @@ def test_gpu_validation_errors(ops):
         ops.backend.gmm(a, b, torch.tensor([3, 6]))                       # sums past the rows of a
     with pytest.raises(RuntimeError):
         ops.backend.gmm(a, b, bs, c=torch.zeros(8, 32, dtype=torch.bfloat16, device="cuda"))
-    with pytest.raises(RuntimeError, match="multiples of 8"):
-        ops.backend.gmm(a[:, :12].contiguous(), b[:, :12].contiguous(), bs)
     with pytest.raises(AssertionError):
         ops.backend.gmm(a, b, bs, trans_a=True, trans_b=True)
 

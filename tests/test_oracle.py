@@ -84,6 +84,16 @@ def test_tolerance_scales_with_the_data(oracle):
     assert oracle.atol_for(torch.full((8, 8), 50.0)) == 1e-2
 
 
+def test_float8_decode_known_values():
+    # the oracle for fp8 operands is the per-expert loop on torch's fp32 decode of the bytes; pin the
+    # decode on values fixed by the OCP formats (1.0, the largest finite value, the smallest
+    # subnormal, a negative value), so that the fnuz variants or a wrong bias would fail
+    e4 = torch.tensor([0x38, 0x7E, 0x01, 0xB8, 0x40], dtype=torch.uint8).view(torch.float8_e4m3fn).float()
+    assert e4.tolist() == [1.0, 448.0, 2.0 ** -9, -1.0, 2.0]
+    e5 = torch.tensor([0x3C, 0x7B, 0x01, 0xBC, 0x40], dtype=torch.uint8).view(torch.float8_e5m2).float()
+    assert e5.tolist() == [1.0, 57344.0, 2.0 ** -16, -1.0, 2.0]
+
+
 def test_zero_k_known_answer(oracle):
     # grouped_gemm/ops_test.py:143-158: ones x ones over k rows is exactly k
     a = torch.ones(192, 128, dtype=torch.bfloat16)
