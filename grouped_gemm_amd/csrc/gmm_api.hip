@@ -18,7 +18,7 @@ const GenericOps* generic_ops_0();
 const GenericOps* generic_ops_1();
 const GenericOps* generic_ops_2();
 const GenericOps* generic_ops_3();
-#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_) const VariantOps* variant_ops_##index();
+#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_, INDEXED_) const VariantOps* variant_ops_##index();
 #include "gmm_variants.def"
 #undef GG_VARIANT
 }  // namespace gg
@@ -46,7 +46,7 @@ int fail(int code, const char* fmt, ...) {
   } while (0)
 
 const gg::VariantOps* (*const kVariantGetters[])() = {
-#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_) &gg::variant_ops_##index,
+#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_, INDEXED_) &gg::variant_ops_##index,
 #include "gmm_variants.def"
 #undef GG_VARIANT
 };
@@ -64,10 +64,12 @@ const gg::GenericOps* generic_ops(int dt) {
   }
 }
 
-const gg::VariantOps* find_variant(int dt, int layout, int shape, int epilogue) {
+const gg::VariantOps* find_variant(int dt, int layout, int shape, int epilogue, int indexed) {
   for (int i = 0; i < kNumVariants; ++i) {
     const gg::VariantOps* v = kVariantGetters[i]();
-    if (v->dt == dt && v->layout == layout && v->shape == shape && v->epilogue == epilogue) return v;
+    if (v->dt == dt && v->layout == layout && v->shape == shape && v->epilogue == epilogue &&
+        v->indexed == indexed)
+      return v;
   }
   return nullptr;
 }
@@ -171,6 +173,14 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   if (g.dtype < GG_DTYPE_BF16 || g.dtype > GG_DTYPE_F8E5M2)
     return fail(GG_EINVAL, "dtype must be one of GG_DTYPE_*");
   const int elem_bytes = g.dtype == GG_DTYPE_F8E4M3 || g.dtype == GG_DTYPE_F8E5M2 ? 1 : 2;
+  if (g.epilogue != GG_EPILOGUE_NONE && g.epilogue != GG_EPILOGUE_SWIGLU)
+    return fail(GG_EINVAL, "epilogue must be one of GG_EPILOGUE_*");
+  const bool swiglu = g.epilogue == GG_EPILOGUE_SWIGLU;
+  if (swiglu && (trans_a || out_f32))
+    return fail(GG_EINVAL, "the SwiGLU epilogue is for the layouts with a row of c per token and a c of the element type");
+  if (swiglu && hidden_in * hidden_out >= (int64_t(1) << 28))
+    return fail(GG_ELIMIT, "hidden_in * hidden_out must be below 2^28 with the SwiGLU epilogue");
+  if (g.a_num_rows < 0 || g.c_num_rows < 0) return fail(GG_EINVAL, "negative row count");
   if (trans_a && g.c_row_index != nullptr)
     return fail(GG_EINVAL, "c_row_index scatters output rows; the trans_a output has none per token");
   if (!trans_a && g.b_row_index != nullptr)
@@ -191,8 +201,13 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   // The streaming kernels fetch and store rows 16 bytes at a time: two-byte elements, hidden sizes
   // that are multiples of 8, operands on 16-byte boundaries, rows in place.  Everything else goes
   // to the kernels of gmm_generic.hpp, VEC elements at a time.
+  const bool indexed = g.a_row_index != nullptr || g.b_row_index != nullptr || g.c_row_index != nullptr;
+  const int64_t a_bytes = (g.a_num_rows > 0 ? g.a_num_rows : tokens) * hidden_in * 2;
+  const int64_t c_bytes = (g.c_num_rows > 0 ? g.c_num_rows : tokens) * hidden_out * 2;
+  // with row indices the streaming kernels address a and c through 32-bit byte offsets
+  const bool indexed_fits = !trans_a && a_bytes < (int64_t)gg::kOutOfRangeIndexed && c_bytes < (int64_t)gg::kOutOfRangeIndexed;
   const bool generic = elem_bytes != 2 || hidden_in % 8 != 0 || hidden_out % 8 != 0 || (address_bits & 15) ||
-                       g.a_row_index != nullptr || g.b_row_index != nullptr || g.c_row_index != nullptr;
+                       (indexed && !indexed_fits);
   int vec = 8;
   if (generic) {
     while (vec > 1 && (hidden_in % vec != 0 || hidden_out % vec != 0 || (address_bits & (uintptr_t)(vec * 2 - 1))))
@@ -215,13 +230,15 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   if (rc != GG_OK) return rc;
   hipStream_t stream = static_cast<hipStream_t>(g.stream);
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
-  const bool short_shape = !generic && use_short_shape(num_groups, tokens, trans_a);
+  const int epilogue = out_f32 ? gg::kEpiAccF32 : (swiglu ? gg::kEpiSwiGLU : gg::kEpiStore);
+  // (the short tile shape exists for the plain epilogue with rows in place only)
+  const bool short_shape = !generic && !swiglu && !indexed && use_short_shape(num_groups, tokens, trans_a);
   const int bm = generic ? gg::kGenericTileM : (short_shape ? Short::BM : Wide::BM);
-  const int bn = generic ? gg::kGenericTileN : (short_shape ? Short::BN : Wide::BN);
+  // output columns per tile: half the tile's width when it holds gate and up columns
+  const int bn = (generic ? gg::kGenericTileN : (short_shape ? Short::BN : Wide::BN)) / (swiglu ? 2 : 1);
   const gg::VariantOps* variant = nullptr;
   if (!generic) {
-    variant = find_variant(g.dtype, layout, short_shape ? Short::kId : Wide::kId,
-                           out_f32 ? gg::kEpiAccF32 : gg::kEpiStore);
+    variant = find_variant(g.dtype, layout, short_shape ? Short::kId : Wide::kId, epilogue, indexed ? 1 : 0);
     if (variant == nullptr) return fail(GG_EINVAL, "no kernel for this combination of arguments");
   }
 
@@ -232,6 +249,11 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   p.tokens = tokens;
   p.hidden_in = (int32_t)hidden_in;
   p.hidden_out = (int32_t)hidden_out;
+  p.b_cols = (int32_t)(swiglu ? 2 * hidden_out : hidden_out);
+  p.a_rows = g.a_row_index;
+  p.c_rows = g.c_row_index;
+  p.a_bytes = (uint32_t)(indexed_fits ? a_bytes : 0);
+  p.c_bytes = (uint32_t)(indexed_fits ? c_bytes : 0);
   p.group_m = band_height(num_groups, tokens, trans_a);
   static_assert(GG_FLAG_WHOLE_TILES == gg::kFlagWholeTiles && GG_FLAG_ONE_CLASS == gg::kFlagOneClass &&
                 GG_FLAG_ROW_PIECES == gg::kFlagRowPieces, "the header's flags are the kernel's");
@@ -244,7 +266,8 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
       return fail(GG_ELIMIT, "the static scratch serves launches of up to %d workgroups, this device has %d "
                   "compute units", kStaticScratchGrid, info.cus);
     p.workspace = reinterpret_cast<char*>(info.scratch);
-    p.ws_slots = (int32_t)(((uint64_t)GG_WORKSPACE_BYTES - gg::kWsCounterBytes) / ((uint64_t)bm * bn * 4));
+    p.ws_slots = (int32_t)(((uint64_t)GG_WORKSPACE_BYTES - gg::kWsCounterBytes) /
+                           ((uint64_t)bm * bn * (swiglu ? 2 : 1) * 4));
     if (p.ws_slots > 1024) p.ws_slots = 1024;
     // Every call on this device shares the array and finds what the last call left: the arrival
     // counters must start at zero (a fill kernel, not a memset: callers may be capturing a graph).
@@ -254,7 +277,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   } else if (g.workspace != nullptr && !generic) {
     if (reinterpret_cast<uintptr_t>(g.workspace) & 255)
       return fail(GG_ELIMIT, "the workspace must be 256-byte aligned");
-    const uint64_t slot_bytes = (uint64_t)bm * bn * 4;
+    const uint64_t slot_bytes = (uint64_t)bm * bn * (swiglu ? 2 : 1) * 4;
     if (g.workspace_bytes < gg::kWsCounterBytes + slot_bytes)
       return fail(GG_ELIMIT, "the workspace holds %llu bytes, the smallest useful one %llu",
                   (unsigned long long)g.workspace_bytes, (unsigned long long)(gg::kWsCounterBytes + slot_bytes));
@@ -307,7 +330,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
       gp.c_rows = g.c_row_index;
       // light workgroups (28 KiB of LDS): two per compute unit
       const int64_t grid = tiles < 2 * info.cus ? tiles : 2 * info.cus;
-      GG_HIP(generic_ops(g.dtype)->launch(layout, vec, out_f32, gp, hs, (int)grid, stream));
+      GG_HIP(generic_ops(g.dtype)->launch(layout, vec, epilogue, gp, hs, (int)grid, stream));
     } else {
       GG_HIP(variant->launch(p, hs, info.cus, stream));
     }
@@ -401,6 +424,7 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   p.hidden_out = (int32_t)hidden_out;
   p.group_m = band_height(num_groups, tokens, trans_a);
   p.num_groups = (int32_t)num_groups;
+  p.b_cols = (int32_t)hidden_out;
   p.sched_out = table_out;
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
   const bool short_shape = use_short_shape(num_groups, tokens, trans_a);

@@ -62,7 +62,10 @@ __device__ __forceinline__ f32x16 mfma(typename Frag<ElemTraits<DT>::BYTES>::typ
 // One operand tile: ROWS indices i (rows of A, columns of B) by BK depth values k.  In memory the
 // element (i, k) sits at base + i * stride_i + k * stride_k (elements), one of the strides being 1;
 // `rows` optionally redirects the index of the strided dimension through an index array.
-template <int ES, int VEC, bool K_CONTIGUOUS>
+// GATE_UP (B with gate | up columns): the tile's 128 indices are 32-index blocks taken alternately
+// from the gate columns [0, out_cols) and the up columns [out_cols, 2 out_cols); i0 and i_end then
+// count output columns.
+template <int ES, int VEC, bool K_CONTIGUOUS, bool GATE_UP = false>
 struct TileLoader {
   static constexpr int VECS = BM * BK / VEC;         // vectors per tile
   static constexpr int PER_THREAD = VECS / THREADS;
@@ -74,6 +77,7 @@ struct TileLoader {
   int k_end;             // the group's depth
   const int32_t* index;  // rows of the strided dimension in memory, or nullptr
   int index_base;        // position of the group's first row in `index`
+  int out_cols;          // GATE_UP: output columns of the group
 
   uint32_t regs[PER_THREAD][VEC * ES > 4 ? VEC * ES / 4 : 1];
 
@@ -93,10 +97,17 @@ struct TileLoader {
     for (int n = 0; n < PER_THREAD; ++n) {
       int i, k;
       coords(threadIdx.x + n * THREADS, &i, &k);
-      const int gi = i0 + i, gk = k0 + k;
+      int gi = i0 + i;
+      const int gk = k0 + k;
+      bool inside = gi < i_end;
+      if constexpr (GATE_UP) {
+        const int block = i >> 5, out = i0 + (block >> 1) * 32 + (i & 31);
+        inside = out < i_end;
+        gi = (block & 1) * out_cols + out;
+      }
 #pragma unroll
       for (int w = 0; w < (VEC * ES > 4 ? VEC * ES / 4 : 1); ++w) regs[n][w] = 0;
-      if (gi < i_end && gk < k_end) {   // extents are multiples of VEC: a vector is all in or all out
+      if (inside && gk < k_end) {   // extents are multiples of VEC: a vector is all in or all out
         int64_t strided = K_CONTIGUOUS ? gi : gk;
         if (index != nullptr) strided = index[index_base + strided];
         const char* src = base + (strided * ld + (K_CONTIGUOUS ? gk : gi)) * ES;
@@ -158,9 +169,11 @@ struct TileLoader {
 
 // DT element type; VEC elements per memory access; the output is c in ElemTraits<DT>::OUT_DT, or
 // fp32 added to when ACC_F32.
-template <int DT, int LAYOUT, int VEC, bool ACC_F32>
+template <int DT, int LAYOUT, int VEC, int EPI>
 __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, HostSizes hs) {
 #if defined(__HIP_DEVICE_COMPILE__)
+  constexpr bool ACC_F32 = EPI == kEpiAccF32, GATE_UP = EPI == kEpiSwiGLU;
+  constexpr int BNS = GATE_UP ? BN / 2 : BN;   // output columns per tile
   constexpr int ES = ElemTraits<DT>::BYTES;
   constexpr int OUT_DT = ElemTraits<DT>::OUT_DT;
   constexpr int PITCH = (BK + PAD) * ES;
@@ -170,7 +183,7 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
   __shared__ Sched sched;
   __shared__ __attribute__((aligned(16))) char tile_a[BM * PITCH];
   __shared__ __attribute__((aligned(16))) char tile_b[BN * PITCH];
-  build_schedule<LAYOUT, BM, BN>(&sched, p, hs);
+  build_schedule<LAYOUT, BM, BNS>(&sched, p, hs);
   __syncthreads();
 
   const int lane = threadIdx.x & 63;
@@ -183,10 +196,10 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
   plan.by_depth = false;
 
   TileLoader<ES, VEC, LAYOUT != kTN> aload;
-  TileLoader<ES, VEC, LAYOUT == kNT> bload;
+  TileLoader<ES, VEC, LAYOUT == kNT, GATE_UP> bload;
   TileCursor cur;
   for (int t = blockIdx.x; t < plan.total; t += gridDim.x) {
-    const TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(&sched, p, t, plan, cur);
+    const TileInfo ti = find_tile<LAYOUT, BM, BNS, BK>(&sched, p, t, plan, cur);
     const int group_row = (int)(ti.g.a_off / p.hidden_in);   // first row of the group in `a`
     // A: NN / NT rows of `a` (depth contiguous); weight gradient: columns of a^T (rows contiguous)
     if (LAYOUT != kTN) {
@@ -212,8 +225,9 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
       bload.index = nullptr;
       bload.index_base = 0;
     }
-    bload.ld = LAYOUT == kNT ? ti.g.k : ti.g.n;
+    bload.ld = LAYOUT == kNT ? ti.g.k : (GATE_UP ? 2 * ti.g.n : ti.g.n);
     bload.i0 = ti.n0, bload.i_end = ti.g.n;
+    bload.out_cols = ti.g.n;
     bload.k_end = ti.depth;
 
     f32x16 acc[2][2];
@@ -264,6 +278,21 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
       int64_t mem_row = row;
       if (gp.c_rows) mem_row = gp.c_rows[out_row0 + row];
       char* crow = cbase + mem_row * ti.g.n * CE;
+      if constexpr (GATE_UP) {
+        // blocks 0 and 1 of the wave hold the gate and the up value of the same 32 output columns
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int col = ti.n0 + wn * 32 + 8 * q + 4 * (lane >> 5);
+          uint16_t* dst = reinterpret_cast<uint16_t*>(crow) + col;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float gate = acc[i][0][4 * q + r], up = acc[i][1][4 * q + r];
+            const u32x2 one = round4<OUT_DT>(gate / (1.0f + __expf(-gate)) * up, 0.0f, 0.0f, 0.0f);
+            if (col + r < ti.g.n) dst[r] = (uint16_t)one[0];
+          }
+        }
+        continue;
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll

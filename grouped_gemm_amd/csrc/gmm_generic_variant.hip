@@ -14,32 +14,37 @@ namespace {
 
 constexpr int DT = GG_GENERIC_DT;
 
-template <int LAYOUT, int VEC, bool ACC_F32>
+template <int LAYOUT, int VEC, int EPI>
 hipError_t launch_one(const GenericParams& gp, const HostSizes& hs, int grid, hipStream_t stream) {
-  hipLaunchKernelGGL((generic::gmm_generic_kernel<DT, LAYOUT, VEC, ACC_F32>), dim3(grid),
+  hipLaunchKernelGGL((generic::gmm_generic_kernel<DT, LAYOUT, VEC, EPI>), dim3(grid),
                      dim3(generic::THREADS), 0, stream, gp, hs);
   return hipGetLastError();
 }
 
-template <int LAYOUT, bool ACC_F32>
+template <int LAYOUT, int EPI>
 hipError_t launch_vec(int vec, const GenericParams& gp, const HostSizes& hs, int grid, hipStream_t stream) {
   switch (vec) {
-    case 8: return launch_one<LAYOUT, 8, ACC_F32>(gp, hs, grid, stream);
-    case 4: return launch_one<LAYOUT, 4, ACC_F32>(gp, hs, grid, stream);
-    case 2: return launch_one<LAYOUT, 2, ACC_F32>(gp, hs, grid, stream);
-    default: return launch_one<LAYOUT, 1, ACC_F32>(gp, hs, grid, stream);
+    case 8: return launch_one<LAYOUT, 8, EPI>(gp, hs, grid, stream);
+    case 4: return launch_one<LAYOUT, 4, EPI>(gp, hs, grid, stream);
+    case 2: return launch_one<LAYOUT, 2, EPI>(gp, hs, grid, stream);
+    default: return launch_one<LAYOUT, 1, EPI>(gp, hs, grid, stream);
   }
 }
 
-hipError_t launch(int layout, int vec, bool acc_f32, const GenericParams& gp, const HostSizes& hs, int grid,
+hipError_t launch(int layout, int vec, int epilogue, const GenericParams& gp, const HostSizes& hs, int grid,
                   hipStream_t stream) {
   if (layout == kTN) {
-    return acc_f32 ? launch_vec<kTN, true>(vec, gp, hs, grid, stream)
-                   : launch_vec<kTN, false>(vec, gp, hs, grid, stream);
+    if (epilogue == kEpiSwiGLU) return hipErrorInvalidValue;
+    return epilogue == kEpiAccF32 ? launch_vec<kTN, kEpiAccF32>(vec, gp, hs, grid, stream)
+                                  : launch_vec<kTN, kEpiStore>(vec, gp, hs, grid, stream);
   }
-  if (acc_f32) return hipErrorInvalidValue;
-  return layout == kNN ? launch_vec<kNN, false>(vec, gp, hs, grid, stream)
-                       : launch_vec<kNT, false>(vec, gp, hs, grid, stream);
+  if (epilogue == kEpiAccF32) return hipErrorInvalidValue;
+  if (epilogue == kEpiSwiGLU) {
+    return layout == kNN ? launch_vec<kNN, kEpiSwiGLU>(vec, gp, hs, grid, stream)
+                         : launch_vec<kNT, kEpiSwiGLU>(vec, gp, hs, grid, stream);
+  }
+  return layout == kNN ? launch_vec<kNN, kEpiStore>(vec, gp, hs, grid, stream)
+                       : launch_vec<kNT, kEpiStore>(vec, gp, hs, grid, stream);
 }
 
 const GenericOps kOps = {DT, &launch};

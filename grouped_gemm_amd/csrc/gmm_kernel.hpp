@@ -59,6 +59,18 @@ struct GmmParams {
   int32_t group_m;     // tile rows per band of the in-group tile order
   int32_t flags;       // kFlag* bits
   int32_t ws_slots;    // partial-tile slots the workspace holds (0: no depth pieces)
+  int32_t b_cols;      // columns of one group's b in memory: hidden_out, or twice that for gate | up
+  // the variants with row indices only:
+  const int32_t* a_rows;   // row r of the left operand is row a_rows[r] of a, or nullptr (rows in place)
+  const int32_t* c_rows;   // row r of the output goes to row c_rows[r] of c, or nullptr
+  uint32_t a_bytes;        // bytes of a and of c in memory, below kOutOfRangeIndexed
+  uint32_t c_bytes;
+};
+
+enum : int {
+  kEpiStore = 0,    // c in the operands' element type, overwritten
+  kEpiAccF32 = 1,   // c in fp32, added to (weight-gradient layout only)
+  kEpiSwiGLU = 2,   // b holds gate | up columns; c = silu(a @ gate) * (a @ up), half as wide
 };
 
 enum : int {   // debugging switches, for comparing the ways a call can be scheduled
@@ -91,7 +103,8 @@ struct TailPlan {
   bool by_depth;
 };
 template <int LAYOUT>
-__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmParams& p, int bk) {
+__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmParams& p, int bk,
+                                              bool depth_pieces_allowed = true) {
   TailPlan t;
   const int rest = tiles % grid;
   t.pieces = 1;
@@ -99,7 +112,7 @@ __device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmPara
   if (rest > 0 && 2 * rest <= grid && !(p.flags & kFlagWholeTiles)) {
     int cand = grid / rest;
     cand = cand > kMaxDepthPieces ? kMaxDepthPieces : cand;
-    if (p.ws_slots > 0 && !(p.flags & kFlagRowPieces)) {
+    if (p.ws_slots > 0 && depth_pieces_allowed && !(p.flags & kFlagRowPieces)) {
       if (rest * cand > p.ws_slots) cand = p.ws_slots / rest;
       cand = cand >= 4 ? 4 : cand;
       if (LAYOUT != kTN) {   // the depth is the same for every tile: keep the pieces worth their fix-up
@@ -138,6 +151,8 @@ struct Sched {
 };
 
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor size used here
+// ... and for the descriptors that span a whole tensor (rows reached through an index)
+constexpr uint32_t kOutOfRangeIndexed = 0xfffffff0u;
 constexpr uint32_t kRsrcFlags = 0x00020000u;   // raw buffer, 32-bit data format
 // Cache policy of the output stores: non-temporal.  The output is written once and never read by
 // this kernel, so it should not push operand lines that other tiles still share out of L2.
@@ -353,6 +368,7 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
 struct GroupGeom {
   int64_t a_off, b_off, c_off;
   int32_t m, n, k;
+  int32_t row0;   // first row of the group in a (and in c, unless c is the weight gradient)
 };
 
 // `e` is the group's index among all groups of the call; `start` and `rows` are the group's
@@ -362,6 +378,7 @@ __device__ __forceinline__ GroupGeom group_geometry(const GmmParams& p, int e, i
                                                     int rows) {
   GroupGeom g;
   const int64_t hin = p.hidden_in, hout = p.hidden_out;
+  g.row0 = (int32_t)start;
   if (LAYOUT == kTN) {
     g.m = p.hidden_in;
     g.n = p.hidden_out;
@@ -374,7 +391,7 @@ __device__ __forceinline__ GroupGeom group_geometry(const GmmParams& p, int e, i
     g.n = p.hidden_out;
     g.k = p.hidden_in;
     g.a_off = start * hin;
-    g.b_off = (int64_t)e * hin * hout;
+    g.b_off = (int64_t)e * hin * p.b_cols;
     g.c_off = start * hout;
   }
   return g;
@@ -437,7 +454,11 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSize
 // A lane's LDS slot is fixed by the hardware (wave base + lane * 16), so the swizzle is
 // applied by choosing which global chunk each lane fetches.
 
-template <int R, int BK, int NT>
+// GATHER: rows come through an index (or in place) at byte offsets kept per load, relative to
+// the start of the whole tensor.  GATE_UP (B of the NT layout with gate | up rows): the tile's R
+// rows are 32-row blocks taken alternately from the gate rows and, `up_step` bytes further, the
+// up rows of b, so that a wave finds the gate and the up value of an output column side by side.
+template <int R, int BK, int NT, bool GATHER = false, bool GATE_UP = false>
 struct DepthMajor {
   static constexpr int CPR = BK / 8;                                  // chunks per row
   static constexpr int RP = (BK * 2 >= 256) ? 1 : 256 / (BK * 2);     // rows per 256 B
@@ -453,6 +474,9 @@ struct DepthMajor {
   int depth;          // depth extent
   int my_chunk;       // depth chunk (of 8) this lane fetches
   uint32_t voff0;     // byte offset of this lane's chunk for load 0
+  uint32_t vrow[GATHER ? NI : 1];   // GATHER: byte offset of this lane's chunk per load
+  uint32_t total_bytes;             // GATHER: bytes of the whole tensor
+  uint32_t up_step;                 // GATE_UP: bytes from a gate row to its up row
 
   __device__ __forceinline__ void setup(const char* tile_base, int ld_, int rows_valid_, int depth_) {
     base = tile_base;
@@ -465,6 +489,40 @@ struct DepthMajor {
     voff0 = (uint32_t)(row * ld + my_chunk * 8) * 2u;
   }
 
+  // GATHER: the tile's row r is row rows[r] of the tensor at `tensor_base` when `rows` is given,
+  // row first_row + r otherwise; rows past rows_valid_ are out of range.
+  __device__ __forceinline__ void setup_gather(const char* tensor_base, uint32_t tensor_bytes,
+                                               const int32_t* rows, int first_row, int ld_,
+                                               int rows_valid_, int depth_) {
+    base = tensor_base;
+    ld = ld_;
+    span = 0;
+    depth = depth_;
+    total_bytes = tensor_bytes;
+    const int tid = threadIdx.x;
+    const int row = tid / CPR, pos = tid % CPR;
+    my_chunk = pos ^ ((row / RP) % CPR);
+    voff0 = 0;
+#pragma unroll
+    for (int i = 0; i < (GATHER ? NI : 1); ++i) {
+      const int r = row + i * ROWS_PER_INSTR;
+      uint32_t v = kOutOfRangeIndexed;
+      if (r < rows_valid_) {
+        const uint32_t src = rows != nullptr ? (uint32_t)rows[r] : (uint32_t)(first_row + r);
+        v = (src * (uint32_t)ld_ + (uint32_t)(my_chunk * 8)) * 2u;
+      }
+      vrow[i] = v;
+    }
+  }
+
+  // GATE_UP: `tile_base` is the tile's first gate row; rows_valid_ counts rows to the end of the
+  // up rows of the group, so that the descriptor ends where the group's b ends.
+  __device__ __forceinline__ void setup_gate_up(const char* tile_base, int ld_, int rows_valid_, int depth_,
+                                                int out_cols) {
+    setup(tile_base, ld_, rows_valid_, depth_);
+    up_step = (uint32_t)out_cols * (uint32_t)ld_ * 2u;
+  }
+
   // Fetch depth slice [kt*BK, kt*BK+BK) into the LDS tile at `dst` (wave-uniform).
   // What all loads of depth slice kt share.
   struct Slice {
@@ -473,17 +531,34 @@ struct DepthMajor {
   };
   __device__ __forceinline__ Slice slice(int kt) const {
     const int left = uniform(depth - kt * BK);
-    const int elems = left > 0 ? span + left : 0;
     Slice sl;
-    sl.rsrc = make_rsrc_words(base + (int64_t)kt * (BK * 2), elems > 0 ? (uint32_t)elems * 2u : 0u);
-    sl.v0 = (left >= BK || my_chunk * 8 < left) ? voff0 : kOutOfRange;
+    if constexpr (GATHER) {
+      // the descriptor spans the tensor from this slice's first byte on; v0 is 0 for a chunk
+      // inside the depth and out of range for one past it
+      const uint32_t skip = (uint32_t)kt * (BK * 2);
+      sl.rsrc = make_rsrc_words(base + skip, left > 0 && total_bytes > skip ? total_bytes - skip : 0u);
+      sl.v0 = (left >= BK || my_chunk * 8 < left) ? 0u : kOutOfRangeIndexed;
+    } else {
+      const int elems = left > 0 ? span + left : 0;
+      sl.rsrc = make_rsrc_words(base + (int64_t)kt * (BK * 2), elems > 0 ? (uint32_t)elems * 2u : 0u);
+      sl.v0 = (left >= BK || my_chunk * 8 < left) ? voff0 : kOutOfRange;
+    }
     return sl;
   }
   // Load I of the NI that make up one slice, into the LDS tile at `dst` (wave-uniform).
   template <int I>
   __device__ __forceinline__ void load(const Slice& sl, const char* dst, int wave) const {
     const uint32_t step = (uint32_t)(ROWS_PER_INSTR * ld) * 2u;
-    load_to_lds_16(sl.rsrc, sl.v0 + I * step, uniform(lds_address(dst) + (I * NT + wave * 64) * 16));
+    uint32_t v;
+    if constexpr (GATHER) {
+      v = vrow[I] | sl.v0;   // either flag pushes the offset out of range
+    } else if constexpr (GATE_UP) {
+      static_assert(ROWS_PER_INSTR == 32, "one load instruction per 32-row block");
+      v = sl.v0 + (I / 2) * step + (I % 2) * up_step;
+    } else {
+      v = sl.v0 + I * step;
+    }
+    load_to_lds_16(sl.rsrc, v, uniform(lds_address(dst) + (I * NT + wave * 64) * 16));
   }
 };
 
@@ -520,6 +595,27 @@ struct WidthMajor {
       const int c = (((p >> 2) ^ seg_swizzle(krow)) << 2) | (p & 3);
       const int col = col0 + c * 8;
       voff[i] = col < width ? (uint32_t)(krow * ld + col) * 2u : kOutOfRange;
+    }
+  }
+
+  // B of the NN layout with gate | up columns: the tile's W columns are 32-column blocks taken
+  // alternately from the gate columns [0, out_cols) and the up columns [out_cols, 2 out_cols) of
+  // the group's b; col0 is the tile's first output column, ld_ = 2 * out_cols.
+  __device__ __forceinline__ void setup_gate_up(const char* group_base, int ld_, int depth_, int col0,
+                                                int out_cols) {
+    base = group_base;
+    ld = ld_;
+    depth = depth_;
+    const int tid = threadIdx.x;
+    const int krow0 = tid / CPRW, p = tid % CPRW;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int krow = krow0 + i * ROWS_PER_INSTR;
+      const int c = (((p >> 2) ^ seg_swizzle(krow)) << 2) | (p & 3);   // 16-byte chunk of the tile row
+      const int block = c >> 2;                                        // 32-column block of the tile
+      const int out = col0 + (block >> 1) * 32 + (c & 3) * 8;          // output column it belongs to
+      const int col = (block & 1) * out_cols + out;
+      voff[i] = out < out_cols ? (uint32_t)(krow * ld + col) * 2u : kOutOfRange;
     }
   }
 
@@ -659,7 +755,7 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   ti.piece = 0;
   ti.rank = 0;
   if (t >= plan.total) {
-    ti.g = GroupGeom{0, 0, 0, 0, 0, 0};
+    ti.g = GroupGeom{0, 0, 0, 0, 0, 0, 0};
     ti.m0 = ti.n0 = ti.rows_valid = ti.depth = 0;
     ti.blocks = 1;
     ti.nk = 1;
@@ -735,17 +831,24 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   return ti;
 }
 
-// ACC_F32: c holds fp32 and the product is added to it (gradient accumulation); otherwise c
-// holds bf16 and is overwritten.
-// DT: element type of a and b (and of c unless ACC_F32).
+// DT: element type of a and b (and of c unless it is the fp32 accumulator).
+// EPI: what happens to a finished tile (kEpi*): stored in the element type; added to an fp32 c
+// (gradient accumulation, weight-gradient layout); or, with gate | up columns in b, combined to
+// silu(gate) * up and stored half as wide.
+// INDEXED: rows of a are fetched and rows of c stored through p.a_rows / p.c_rows (NN and NT).
 template <int DT, int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N,
-          bool ACC_F32 = false>
+          int EPI = kEpiStore, bool INDEXED = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p, HostSizes hs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
   constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB, KS = BK / 16;
-  using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT>, WidthMajor<BM, BK, NT>>;
-  using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT>, WidthMajor<BN, BK, NT>>;
+  constexpr bool ACC_F32 = EPI == kEpiAccF32, GATE_UP = EPI == kEpiSwiGLU;
+  static_assert(!ACC_F32 || LAYOUT == kTN, "the fp32 accumulator is the weight gradient's");
+  static_assert(!(GATE_UP || INDEXED) || LAYOUT != kTN, "row indices and gate | up are for the NN and NT layouts");
+  static_assert(!GATE_UP || NB % 2 == 0, "a wave needs the gate and the up block of its columns");
+  constexpr int BNS = GATE_UP ? BN / 2 : BN;   // output columns per tile, what the schedule counts in
+  using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT, INDEXED>, WidthMajor<BM, BK, NT>>;
+  using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT, false, GATE_UP>, WidthMajor<BN, BK, NT>>;
   using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK, WAVES_M>, WidthMajorFrag<BM, BK, MB, WAVES_M>>;
   using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK, 1>, WidthMajorFrag<BN, BK, NB, 1>>;
   constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;   // per lane, per depth slice
@@ -756,7 +859,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   Sched* sched = reinterpret_cast<Sched*>(smem + Cfg::SCHED_OFFSET);
-  build_schedule<LAYOUT, BM, BN>(sched, p, hs);
+  build_schedule<LAYOUT, BM, BNS>(sched, p, hs);
   __syncthreads();
 
   const int lane = threadIdx.x & 63;
@@ -768,9 +871,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   afrag.setup(wm * 32);   // wave row wm owns row blocks wm, wm + WAVES_M, ...
   bfrag.setup(wn * Cfg::WTN);
 
+  // (a tile that is combined or scattered on its way out is never cut along the depth: the
+  // fix-up of the depth pieces stores plain tiles)
   const TailPlan plan = plan_tail<LAYOUT>(
       uniform(sched->tile_start[p.num_groups]) + uniform(sched->runt_start[p.num_groups]),
-      (int)gridDim.x, p, BK);
+      (int)gridDim.x, p, BK, !(GATE_UP || INDEXED));
   const int total_tiles = plan.total;
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
@@ -789,14 +894,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   TileCursor fetch_cur;
   TileInfo fti;
   auto fetch_setup = [&]() {
-    fti = find_tile<LAYOUT, BM, BN, BK>(sched, p, fetch_t, plan, fetch_cur);
+    fti = find_tile<LAYOUT, BM, BNS, BK>(sched, p, fetch_t, plan, fetch_cur);
     const int depth = fti.depth;
-    if constexpr (Cfg::A_DEPTH_MAJOR) {
+    if constexpr (INDEXED) {
+      const int first = fti.g.row0 + fti.m0;
+      aload.setup_gather(p.a, p.a_bytes, p.a_rows != nullptr ? p.a_rows + first : nullptr, first, fti.g.k,
+                         depth > 0 ? fti.rows_valid : 0, depth);
+    } else if constexpr (Cfg::A_DEPTH_MAJOR) {
       aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * 2, fti.g.k, fti.rows_valid, depth);
     } else {
       aload.setup(p.a + fti.g.a_off * 2, fti.g.m, depth, fti.m0, fti.g.m);
     }
-    if constexpr (Cfg::B_DEPTH_MAJOR) {
+    if constexpr (GATE_UP && Cfg::B_DEPTH_MAJOR) {
+      bload.setup_gate_up(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
+                          fti.valid && depth > 0 ? 2 * fti.g.n - fti.n0 : 0, depth, fti.g.n);
+    } else if constexpr (GATE_UP) {
+      bload.setup_gate_up(p.b + fti.g.b_off * 2, 2 * fti.g.n, depth, fti.n0, fti.g.n);
+    } else if constexpr (Cfg::B_DEPTH_MAJOR) {
       bload.setup(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
                   fti.valid && depth > 0 ? min(BN, fti.g.n - fti.n0) : 0, depth);
     } else {
@@ -863,7 +977,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 
   int tile_t = vid;
   TileCursor tile_cur;
-  TileInfo ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_cur);
+  TileInfo ti = find_tile<LAYOUT, BM, BNS, BK>(sched, p, tile_t, plan, tile_cur);
   wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
@@ -981,9 +1095,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     // where it is converted, so the epilogue needs only a few vector registers.
     {
       constexpr int CE = ACC_F32 ? 4 : 2;   // bytes per element of c
-      const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * CE;
-      const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * (uint32_t)CE : 0u;
+      constexpr uint32_t OOR = INDEXED ? kOutOfRangeIndexed : kOutOfRange;
+      // the descriptor covers the tile's rows of c, or all of c when rows go through an index
+      const char* cbase = INDEXED ? p.c : p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * CE;
+      const uint32_t cbytes = INDEXED ? p.c_bytes
+                              : (ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * (uint32_t)CE : 0u);
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
+      // byte offset of row `row` of the tile in that descriptor (OOR: the row does not exist)
+      auto row_offset = [&](int row) -> uint32_t {
+        if constexpr (INDEXED) {
+          if (row >= ti.rows_valid) return OOR;
+          const int r = ti.g.row0 + ti.m0 + row;
+          const uint32_t dst = p.c_rows != nullptr ? (uint32_t)p.c_rows[r] : (uint32_t)r;
+          return dst * (uint32_t)ti.g.n * 2u;
+        } else {
+          return (uint32_t)(row * ti.g.n) * (uint32_t)CE;
+        }
+      };
+      auto at = [&](uint32_t row_off, int col) -> uint32_t {
+        return col < ti.g.n && (!INDEXED || row_off != OOR) ? row_off + (uint32_t)col * (uint32_t)CE : OOR;
+      };
       auto take4 = [&](int i, int j, int q) {
         float v[4];
 #pragma unroll
@@ -991,7 +1122,32 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
           asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[r]) : "a"(acc[i][j][4 * q + r]));
         return round4<DT>(v[0], v[1], v[2], v[3]);
       };
-      if constexpr (ACC_F32) {
+      if constexpr (GATE_UP) {
+        // Blocks 2 jp and 2 jp + 1 of a wave hold the gate and the up value of the same 32 output
+        // columns, element for element: silu(gate) * up in fp32, one rounding, 8 bytes per lane.
+#pragma unroll
+        for (int i = 0; i < ML; ++i) {
+          const uint32_t row_off = row_offset((wm + i * WAVES_M) * 32 + (lane & 31));
+#pragma unroll
+          for (int jp = 0; jp < NB / 2; ++jp) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              float o[4];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                float gate, up;
+                asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(gate) : "a"(acc[i][2 * jp][4 * q + r]));
+                asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(up) : "a"(acc[i][2 * jp + 1][4 * q + r]));
+                o[r] = gate / (1.0f + __expf(-gate)) * up;
+              }
+              const int col = ti.n0 + wn * (Cfg::WTN / 2) + jp * 32 + 8 * q + 4 * (lane >> 5);
+              __builtin_amdgcn_raw_buffer_store_b64(round4<DT>(o[0], o[1], o[2], o[3]), rc, at(row_off, col), 0,
+                                                    kStoreStreaming);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      } else if constexpr (ACC_F32) {
         // c += product in fp32.  The 4 consecutive columns a lane holds are 16 bytes of c:
         // read them, add, write them back; lanes l and l + 32 cover 32 contiguous bytes of a
         // row, four such instructions one 128-byte line.  All reads of a 32-row block row are
@@ -1036,6 +1192,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
         const int out_row = lane >> 3, out_chunk = lane & 7;
 #pragma unroll
         for (int i = 0; i < ML; ++i) {
+          uint32_t row_off[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) row_off[r] = row_offset((wm + i * WAVES_M) * 32 + r * 8 + out_row);
 #pragma unroll
           for (int jp = 0; jp < NB / 2; ++jp) {
 #pragma unroll
@@ -1047,10 +1206,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const u32x4 v = *reinterpret_cast<const u32x4*>(strip + (r * 8 + out_row) * PITCH + out_chunk * 16);
-              const int row = (wm + i * WAVES_M) * 32 + r * 8 + out_row;
               const int col = ti.n0 + wn * Cfg::WTN + jp * 64 + out_chunk * 8;
-              const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
-              __builtin_amdgcn_raw_buffer_store_b128(v, rc, off, 0, kStoreStreaming);
+              __builtin_amdgcn_raw_buffer_store_b128(v, rc, at(row_off[r], col), 0, kStoreStreaming);
             }
             // keep the conversion of one strip from being hoisted over the stores of the
             // previous one: few accumulators are live in vector registers at a time
@@ -1060,14 +1217,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       } else {
 #pragma unroll
         for (int i = 0; i < ML; ++i) {
-          const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
+          const uint32_t row_off = row_offset((wm + i * WAVES_M) * 32 + (lane & 31));
 #pragma unroll
           for (int j = 0; j < NB; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
-              const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 2u : kOutOfRange;
-              __builtin_amdgcn_raw_buffer_store_b64(take4(i, j, q), rc, off, 0, kStoreStreaming);
+              __builtin_amdgcn_raw_buffer_store_b64(take4(i, j, q), rc, at(row_off, col), 0, kStoreStreaming);
             }
             __builtin_amdgcn_sched_barrier(0);
           }
@@ -1095,7 +1251,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     }
     tile_t += G;
     if (tile_t >= total_tiles) break;
-    ti = find_tile<LAYOUT, BM, BN, BK>(sched, p, tile_t, plan, tile_cur);
+    ti = find_tile<LAYOUT, BM, BNS, BK>(sched, p, tile_t, plan, tile_cur);
   }
   wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
 

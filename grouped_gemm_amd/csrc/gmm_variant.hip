@@ -12,10 +12,11 @@ namespace {
 
 template <int INDEX>
 struct VariantDef;
-#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_)                                    \
+#define GG_VARIANT(index, DT_, LAYOUT_, SHAPE_, EPI_, INDEXED_)                          \
   template <>                                                                            \
   struct VariantDef<index> {                                                             \
     static constexpr int DT = DT_, LAYOUT = LAYOUT_, EPI = EPI_;                         \
+    static constexpr bool INDEXED = INDEXED_;                                            \
     using Shape = SHAPE_;                                                                \
   };
 #include "gmm_variants.def"
@@ -27,7 +28,7 @@ using Cfg = GmmConfig<V::LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_
 
 const void* kernel_address() {
   return reinterpret_cast<const void*>(
-      &gmm_kernel<V::DT, V::LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, V::EPI == kEpiAccF32>);
+      &gmm_kernel<V::DT, V::LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, V::EPI, V::INDEXED>);
 }
 
 hipError_t prepare() {
@@ -42,7 +43,7 @@ hipError_t launch(const GmmParams& p, const HostSizes& hs, int grid, hipStream_t
                          Cfg::LDS_BYTES, stream);
 }
 
-const VariantOps kOps = {V::DT, V::LAYOUT, S::kId, V::EPI, Cfg::LDS_BYTES, &prepare, &launch};
+const VariantOps kOps = {V::DT, V::LAYOUT, S::kId, V::EPI, V::INDEXED ? 1 : 0, Cfg::LDS_BYTES, &prepare, &launch};
 
 }  // namespace
 

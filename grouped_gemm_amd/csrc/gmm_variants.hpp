@@ -22,13 +22,8 @@ struct Short {
   static constexpr int kId = 1, BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
 };
 
-enum : int {
-  kEpiStore = 0,    // c in the operands' element type, overwritten
-  kEpiAccF32 = 1,   // c in fp32, added to (weight-gradient layout only)
-};
-
 struct VariantOps {
-  int dt, layout, shape, epilogue;
+  int dt, layout, shape, epilogue, indexed;
   int lds_bytes;
   // raises the kernel's dynamic LDS limit on the current device
   hipError_t (*prepare)();
@@ -39,7 +34,7 @@ struct VariantOps {
 struct GenericParams;
 struct GenericOps {
   int dt;
-  hipError_t (*launch)(int layout, int vec, bool acc_f32, const GenericParams& gp, const HostSizes& hs,
+  hipError_t (*launch)(int layout, int vec, int epilogue, const GenericParams& gp, const HostSizes& hs,
                        int grid, hipStream_t stream);
 };
 constexpr int kGenericTileM = 128, kGenericTileN = 128;

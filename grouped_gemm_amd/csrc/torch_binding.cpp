@@ -44,9 +44,10 @@ struct RowIndices {
 // rank and dtype rules can be exercised with CPU tensors on a machine without one.
 // With row indices, `tokens` (the rows of the product) is the length of the index instead of the
 // row count of the tensor it redirects.
+// With `gate_up`, b holds two matrices per expert side by side and c is half as wide as b.
 void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
               const torch::Tensor& batch_sizes, bool trans_a, bool trans_b, bool on_device,
-              const RowIndices& rows = RowIndices()) {
+              const RowIndices& rows = RowIndices(), bool gate_up = false) {
   // Only one of the operands may be transposed (csrc/grouped_gemm.cu:476).
   TORCH_CHECK(!(trans_a && trans_b), "grouped_gemm: trans_a and trans_b cannot both be set");
 
@@ -78,6 +79,7 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
     if (on_device) TORCH_CHECK(idx->is_cuda() && idx->device() == a.device(), "grouped_gemm: a row index must be on a's GPU");
   }
   TORCH_CHECK(!(trans_a && rows.c.defined()), "grouped_gemm: the trans_a output has no row per token to scatter");
+  TORCH_CHECK(!(trans_a && gate_up), "grouped_gemm: the SwiGLU epilogue is not for the trans_a layout");
   TORCH_CHECK(trans_a || !rows.b.defined(), "grouped_gemm: only the trans_a layout has a row per token in b");
   const int64_t tokens = rows.a.defined() ? rows.a.size(0) : a.size(0);
 
@@ -101,7 +103,9 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
     TORCH_CHECK(batch_sizes.size(0) == b.size(0), "grouped_gemm: need one batch size per expert");
     // The reference leaves the shape of c unchecked here; a wrong one would make the
     // kernel write outside c, so it is rejected.
-    const int64_t hidden_out = trans_b ? b.size(1) : b.size(2);
+    TORCH_CHECK(!gate_up || (trans_b ? b.size(1) : b.size(2)) % 2 == 0,
+                "grouped_gemm: with gate | up columns, b must hold an even number of them");
+    const int64_t hidden_out = (trans_b ? b.size(1) : b.size(2)) / (gate_up ? 2 : 1);
     if (rows.c.defined()) {
       TORCH_CHECK(rows.c.size(0) == tokens, "grouped_gemm: c_rows needs one entry per row of the product");
       TORCH_CHECK(c.size(1) == hidden_out, "grouped_gemm: c must have hidden_out columns");
@@ -146,7 +150,8 @@ torch::Tensor Workspace(const torch::Device& device, hipStream_t stream) {
 }
 
 void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c, const torch::Tensor& batch_sizes,
-         bool trans_a, bool trans_b, bool accumulate_f32, int64_t flags, const RowIndices& rows = RowIndices()) {
+         bool trans_a, bool trans_b, bool accumulate_f32, int64_t flags, const RowIndices& rows = RowIndices(),
+         bool gate_up = false) {
   torch::Tensor sizes = batch_sizes.is_cpu() ? batch_sizes.contiguous() : batch_sizes;
   c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
@@ -169,7 +174,10 @@ void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
   g.b_row_index = rows.b.defined() ? rows.b.data_ptr<int32_t>() : nullptr;
   g.c_row_index = rows.c.defined() ? rows.c.data_ptr<int32_t>() : nullptr;
   g.hidden_in = a.size(1);
-  g.hidden_out = trans_a ? b.size(1) : (trans_b ? b.size(1) : b.size(2));
+  g.hidden_out = (trans_a ? b.size(1) : (trans_b ? b.size(1) : b.size(2))) / (gate_up ? 2 : 1);
+  g.epilogue = gate_up ? GG_EPILOGUE_SWIGLU : GG_EPILOGUE_NONE;
+  g.a_num_rows = a.size(0);
+  g.c_num_rows = trans_a ? 0 : c.size(0);
   g.workspace = ws.data_ptr();
   g.workspace_bytes = (uint64_t)ws.numel();
   g.flags = (int32_t)flags;
@@ -204,6 +212,16 @@ void GroupedGemmIndexed(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch
   if (c_rows.has_value()) rows.c = *c_rows;
   Validate(a, b, c, batch_sizes, trans_a, trans_b, /*on_device=*/true, rows);
   Run(a, b, c, batch_sizes, trans_a, trans_b, /*accumulate_f32=*/false, /*flags=*/0, rows);
+}
+
+// c = silu(a @ gate) * (a @ up) with b = [gate | up] per expert, optionally with row indices.
+void GroupedGemmSwiGLU(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes, bool trans_b,
+                       c10::optional<torch::Tensor> a_rows, c10::optional<torch::Tensor> c_rows) {
+  RowIndices rows;
+  if (a_rows.has_value()) rows.a = *a_rows;
+  if (c_rows.has_value()) rows.c = *c_rows;
+  Validate(a, b, c, batch_sizes, /*trans_a=*/false, trans_b, /*on_device=*/true, rows, /*gate_up=*/true);
+  Run(a, b, c, batch_sizes, /*trans_a=*/false, trans_b, /*accumulate_f32=*/false, /*flags=*/0, rows, /*gate_up=*/true);
 }
 
 // c (num_experts, hidden_in, hidden_out) fp32 += per expert a_e^T @ b_e; see gg_gmm_bf16_acc_f32.
@@ -249,6 +267,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gmm_indexed", &GroupedGemmIndexed, "gmm with fused row gather / scatter.", py::arg("a"), py::arg("b"),
         py::arg("c"), py::arg("batch_sizes"), py::arg("trans_a"), py::arg("trans_b"), py::arg("a_rows") = py::none(),
         py::arg("b_rows") = py::none(), py::arg("c_rows") = py::none());
+  m.def("gmm_swiglu", &GroupedGemmSwiGLU, "silu(a @ gate) * (a @ up) with b = [gate | up].", py::arg("a"),
+        py::arg("b"), py::arg("c"), py::arg("batch_sizes"), py::arg("trans_b"), py::arg("a_rows") = py::none(),
+        py::arg("c_rows") = py::none());
   m.def("gmm_with_flags", &GroupedGemmWithFlags, "gmm with GG_FLAG_* bits (testing).");
   m.attr("flag_whole_tiles") = GG_FLAG_WHOLE_TILES;
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,

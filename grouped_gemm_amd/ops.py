@@ -114,6 +114,45 @@ def gmm_scatter(a, w, batch_sizes, row_index, trans_b=False):
     return GroupedGemmScatter.apply(a, w, batch_sizes, row_index, trans_b)
 
 
+# ------------------------------------------------------------------ gated activation
+
+class GroupedGemmSwiGLU(torch.autograd.Function):
+    """silu(a @ gate) * (a @ up) with w = [gate | up] per expert, the activation fused into the
+    GEMM's epilogue.  The backward recomputes the two products with a plain grouped GEMM (they are
+    not stored by the forward), applies the derivative elementwise and runs the two usual
+    gradient GEMMs on the result."""
+
+    @staticmethod
+    def forward(ctx, a, w, batch_sizes, trans_b):
+        ctx.save_for_backward(a, w, batch_sizes)
+        ctx.trans_b = trans_b
+        return backend.gmm_swiglu(a, w, batch_sizes, trans_b=trans_b)
+
+    @staticmethod
+    def backward(ctx, grad):
+        grad = grad.contiguous()
+        a, w, batch_sizes = ctx.saved_tensors
+        gate_up = backend.gmm(a, w, batch_sizes, trans_b=ctx.trans_b).float()
+        gate, up = gate_up.chunk(2, dim=-1)
+        sig = torch.sigmoid(gate)
+        g32 = grad.float()
+        dgate = g32 * up * sig * (1.0 + gate * (1.0 - sig))
+        dup = g32 * gate * sig
+        dgu = torch.cat([dgate, dup], dim=-1).to(a.dtype)
+        agrad = wgrad = None
+        if ctx.needs_input_grad[0]:
+            agrad = backend.gmm(dgu, w, batch_sizes, trans_b=not ctx.trans_b)
+        if ctx.needs_input_grad[1]:
+            lhs, rhs = (dgu, a) if ctx.trans_b else (a, dgu)
+            wgrad = backend.gmm(lhs, rhs, batch_sizes, trans_a=True)
+        return agrad, wgrad, None, None
+
+
+def gmm_swiglu(a, w, batch_sizes, trans_b=False):
+    """silu(a @ gate) * (a @ up) per expert, w = [gate | up]; see backend.gmm_swiglu."""
+    return GroupedGemmSwiGLU.apply(a, w, batch_sizes, trans_b)
+
+
 # ------------------------------------------------------------------ traceable form
 #
 # The same operator registered with torch.library, so that torch.compile sees one opaque node

@@ -43,6 +43,10 @@ extern "C" {
 #define GG_DTYPE_F8E4M3 2   /* OCP e4m3 (torch.float8_e4m3fn) in a and b, bf16 in c */
 #define GG_DTYPE_F8E5M2 3   /* OCP e5m2 (torch.float8_e5m2) in a and b, bf16 in c */
 
+/* gg_gmm_args.epilogue */
+#define GG_EPILOGUE_NONE 0
+#define GG_EPILOGUE_SWIGLU 1   /* b holds gate | up columns; c = silu(a @ gate) * (a @ up) */
+
 /* Bytes of workspace that let any call cut the tiles of its last, partly filled round along the
  * depth (see gg_gmm): 4096 bytes of arrival counters and 256 partial tiles of 256 x 256 floats. */
 #define GG_WORKSPACE_BYTES (4096 + 256 * 256 * 256 * 4)
@@ -135,6 +139,17 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  *                 c_row_index[r] of c (a scatter fused into the store; not with trans_a).  Rows of
  *                 c that no index names are not touched.  Indices are not checked: each must
  *                 name a row that exists, and c_row_index must not name a row twice.
+ *   a_num_rows, c_num_rows
+ *                 Rows of a and of c in memory when a row index redirects them (0: `tokens`).
+ *                 With two-byte elements, aligned operands and a and c below 4 GiB the NN and NT
+ *                 layouts run indexed on the streaming kernels; otherwise, and with trans_a, on
+ *                 the general ones.
+ *   epilogue      GG_EPILOGUE_SWIGLU (not with trans_a or accumulate_f32): b holds two matrices
+ *                 per group side by side, gate and up: (num_groups, hidden_in, 2 * hidden_out), or
+ *                 (num_groups, 2 * hidden_out, hidden_in) with trans_b, gate first.  c (tokens,
+ *                 hidden_out) = silu(a @ gate) * (a @ up) with silu(x) = x / (1 + exp(-x)), both
+ *                 products accumulated and combined in fp32, rounded once.  The reference has no
+ *                 epilogue hook (alpha = 1, beta = 0, csrc/grouped_gemm.cu:255).
  *   accumulate_f32  1: c is fp32 and is added to (trans_a = 1 only), as gg_gmm_bf16_acc_f32.
  *   workspace, workspace_bytes
  *                 Device memory the call may use for partial results, or NULL.  When the last
@@ -172,6 +187,10 @@ typedef struct gg_gmm_args {
   const int32_t* a_row_index;
   const int32_t* b_row_index;
   const int32_t* c_row_index;
+  int64_t a_num_rows;
+  int64_t c_num_rows;
+  int32_t epilogue;
+  int32_t reserved1;
 } gg_gmm_args;
 
 int gg_gmm(const gg_gmm_args* args);

@@ -11,6 +11,7 @@ Contents
                       csrc/grouped_gemm.cu:418-435.  With dtype=float32 the slices are
                       up-cast first, which gives the fp32-accumulated result the
                       tolerance is stated against.
+  swiglu_loop         the gated activation silu(a @ gate) * (a @ up) on top of that loop.
   gmm_c               same result from the plain-C triple loop in gg_oracle.c
                       (small shapes only).
   table_walk / table_closed / table_numpy
@@ -120,6 +121,19 @@ def gmm_loop(a, b, batch_sizes, trans_a=False, trans_b=False, dtype=torch.float3
                 out[start:start + size] = lhs @ (rhs.t() if trans_b else rhs)
         start += size
     return out
+
+
+def swiglu_loop(a, b, batch_sizes, trans_b=False, dtype=torch.float32):
+    """silu(a_e @ gate_e) * (a_e @ up_e) per expert with b = [gate | up] side by side (gate first):
+    the per-expert loop above on the two halves of b, combined elementwise in `dtype` with
+    silu(x) = x / (1 + exp(-x)).  The products are the pinned loop; the activation is pinned against
+    its closed form at known points in tests/test_oracle.py."""
+    half = (b.shape[1] if trans_b else b.shape[2]) // 2
+    gate_w = b[:, :half] if trans_b else b[:, :, :half]
+    up_w = b[:, half:] if trans_b else b[:, :, half:]
+    gate = gmm_loop(a, gate_w.contiguous(), batch_sizes, trans_b=trans_b, dtype=dtype)
+    up = gmm_loop(a, up_w.contiguous(), batch_sizes, trans_b=trans_b, dtype=dtype)
+    return gate / (1.0 + torch.exp(-gate)) * up
 
 
 def accumulate_weight_gradient_loop(a, b, batch_sizes, c0, dtype=torch.float64):

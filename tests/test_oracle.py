@@ -84,6 +84,31 @@ def test_tolerance_scales_with_the_data(oracle):
     assert oracle.atol_for(torch.full((8, 8), 50.0)) == 1e-2
 
 
+def test_swiglu_loop_known_values(oracle):
+    # one expert, one depth: the products are the inputs themselves, so the result must be the
+    # closed form at points fixed by hand: silu(0) = 0, silu(ln 3) = ln(3) * 3 / 4, silu(-ln 3) =
+    # -ln(3) / 4, large negative gate -> 0, and the up value multiplies it
+    import math
+    ln3 = math.log(3.0)
+    a = torch.ones(1, 1, dtype=torch.bfloat16)
+    for gate, up, want in [(0.0, 5.0, 0.0), (2.0, 1.0, 2.0 / (1.0 + math.exp(-2.0))),
+                           (-2.0, 3.0, -6.0 / (1.0 + math.exp(2.0))), (-60.0, 1.0, 0.0), (4.0, -0.5, -2.0 / (1 + math.exp(-4.0)))]:
+        b = torch.tensor([[[gate, up]]], dtype=torch.bfloat16)               # (1, 1, 2): gate | up
+        got = float(oracle.swiglu_loop(a, b, torch.tensor([1]))[0, 0])
+        assert abs(got - want) <= 1e-6 * max(1.0, abs(want)), (gate, up, got, want)
+    assert abs(ln3 * 0.75 - float(oracle.swiglu_loop(torch.ones(1, 1), torch.tensor([[[ln3, 1.0]]]), torch.tensor([1]))[0, 0])) < 1e-6
+    # trans_b layout: rows of b are columns of the product, gate rows first
+    g = torch.Generator().manual_seed(3)
+    a2 = torch.randn(7, 5, generator=g).to(torch.bfloat16)
+    b2 = torch.randn(2, 5, 6, generator=g).to(torch.bfloat16)
+    bs = torch.tensor([3, 4])
+    nn = oracle.swiglu_loop(a2, b2, bs)
+    nt = oracle.swiglu_loop(a2, b2.transpose(1, 2).contiguous(), bs, trans_b=True)
+    assert nn.shape == (7, 3) and torch.equal(nn, nt)
+    want = torch.nn.functional.silu(oracle.gmm_loop(a2, b2[:, :, :3].contiguous(), bs)) * oracle.gmm_loop(a2, b2[:, :, 3:].contiguous(), bs)
+    torch.testing.assert_close(nn, want, rtol=1e-6, atol=1e-6)
+
+
 def test_float8_decode_known_values():
     # the oracle for fp8 operands is the per-expert loop on torch's fp32 decode of the bytes; pin the
     # decode on values fixed by the OCP formats (1.0, the largest finite value, the smallest
