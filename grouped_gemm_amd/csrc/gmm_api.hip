@@ -206,8 +206,11 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   const int64_t c_bytes = (g.c_num_rows > 0 ? g.c_num_rows : tokens) * hidden_out * 2;
   // with row indices the streaming kernels address a and c through 32-bit byte offsets
   const bool indexed_fits = !trans_a && a_bytes < (int64_t)gg::kOutOfRangeIndexed && c_bytes < (int64_t)gg::kOutOfRangeIndexed;
-  const bool generic = elem_bytes != 2 || hidden_in % 8 != 0 || hidden_out % 8 != 0 || (address_bits & 15) ||
-                       (indexed && !indexed_fits);
+  // (fp8: the NT layout streams, rows of 16-byte chunks again; the other layouts would need
+  // byte-wise transposing reads and go to the general kernels)
+  const bool f8_streams = elem_bytes == 1 && !trans_a && trans_b && hidden_in % 16 == 0 && !indexed && !swiglu;
+  const bool generic = (elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
+                       (address_bits & 15) || (indexed && !indexed_fits);
   int vec = 8;
   if (generic) {
     while (vec > 1 && (hidden_in % vec != 0 || hidden_out % vec != 0 || (address_bits & (uintptr_t)(vec * 2 - 1))))
@@ -231,8 +234,9 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   hipStream_t stream = static_cast<hipStream_t>(g.stream);
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
   const int epilogue = out_f32 ? gg::kEpiAccF32 : (swiglu ? gg::kEpiSwiGLU : gg::kEpiStore);
-  // (the short tile shape exists for the plain epilogue with rows in place only)
-  const bool short_shape = !generic && !swiglu && !indexed && use_short_shape(num_groups, tokens, trans_a);
+  // (the short tile shape exists for two-byte elements, the plain epilogue and rows in place only)
+  const bool short_shape = !generic && !swiglu && !indexed && elem_bytes == 2 &&
+                           use_short_shape(num_groups, tokens, trans_a);
   const int bm = generic ? gg::kGenericTileM : (short_shape ? Short::BM : Wide::BM);
   // output columns per tile: half the tile's width when it holds gate and up columns
   const int bn = (generic ? gg::kGenericTileN : (short_shape ? Short::BN : Wide::BN)) / (swiglu ? 2 : 1);

@@ -16,11 +16,9 @@
 
 namespace gg {
 
-enum : int { kF8E4M3 = 2, kF8E5M2 = 3 };   // one-byte element types (OCP), c is bf16
-
 template <int DT>
 struct ElemTraits {
-  static constexpr int BYTES = (DT == kF8E4M3 || DT == kF8E5M2) ? 1 : 2;
+  static constexpr int BYTES = is_f8(DT) ? 1 : 2;
   static constexpr int OUT_DT = DT == kF16 ? kF16 : kBF16;   // element type of c
 };
 

@@ -30,7 +30,10 @@ constexpr int kMaxGroups = 512;
 constexpr int kSchedCols = 14;
 
 enum : int { kNN = 0, kNT = 1, kTN = 2 };
-enum : int { kBF16 = 0, kF16 = 1 };   // element type of the operands, two bytes either way
+// Element types of a and b.  Two-byte types give a c of the same type; the one-byte (OCP fp8)
+// types give a bf16 c.
+enum : int { kBF16 = 0, kF16 = 1, kF8E4M3 = 2, kF8E5M2 = 3 };
+constexpr bool is_f8(int dt) { return dt == kF8E4M3 || dt == kF8E5M2; }
 
 using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
 using bf16x4 = __attribute__((ext_vector_type(4))) __bf16;
@@ -40,6 +43,8 @@ using f32x16 = __attribute__((ext_vector_type(16))) float;
 using f32x4 = __attribute__((ext_vector_type(4))) float;
 using u32x2 = __attribute__((ext_vector_type(2))) uint32_t;
 using u32x4 = __attribute__((ext_vector_type(4))) uint32_t;
+using i32x4 = __attribute__((ext_vector_type(4))) int;
+using i32x8 = __attribute__((ext_vector_type(8))) int;
 
 #define GG_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
@@ -224,6 +229,18 @@ __device__ __forceinline__ f32x16 mfma_32x32x16(bf16x8 x, bf16x8 y, f32x16 acc) 
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, x),
                                                   __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
   }
+}
+
+// One 32x32x64 matrix instruction on fp8 fragments: 32 one-byte elements per lane and operand,
+// handed over as the two 16-byte halves they are read from LDS in.
+template <int DT>
+__device__ __forceinline__ f32x16 mfma_32x32x64_f8(bf16x8 x_lo, bf16x8 x_hi, bf16x8 y_lo, bf16x8 y_hi, f32x16 acc) {
+  const i32x8 x = __builtin_shufflevector(__builtin_bit_cast(i32x4, x_lo), __builtin_bit_cast(i32x4, x_hi), 0, 1, 2,
+                                          3, 4, 5, 6, 7);
+  const i32x8 y = __builtin_shufflevector(__builtin_bit_cast(i32x4, y_lo), __builtin_bit_cast(i32x4, y_hi), 0, 1, 2,
+                                          3, 4, 5, 6, 7);
+  constexpr int FORMAT = DT == kF8E5M2 ? 1 : 0;   // e4m3 : e5m2, for both operands; no block scales
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, FORMAT, FORMAT, 0, 0, 0, 0);
 }
 
 // Four fp32 values rounded (to nearest even) to the element type, as 8 bytes.
@@ -641,7 +658,10 @@ struct WidthMajor {
 
 // STRIDE: distance between the blocks a wave owns, in 32-wide blocks (the waves along a
 // dimension take blocks alternately when STRIDE is their number, contiguously when it is 1).
-template <int BK, int STRIDE>
+// F8: one-byte elements.  A row of the tile is then 128 depth values, and the fragment of one
+// 32x32x64 instruction is 32 consecutive bytes of it (depth 32 (l / 32) .. +31 of a 64-deep step),
+// read as two 16-byte halves: "step" 2 s + h below is half h of 64-deep step s.
+template <int BK, int STRIDE, bool F8 = false>
 struct DepthMajorFrag {
   static constexpr int CPR = BK / 8;
   static constexpr int RP = (BK * 2 >= 256) ? 1 : 256 / (BK * 2);
@@ -654,7 +674,8 @@ struct DepthMajorFrag {
     const int sw = (row / RP) % CPR;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      off[ks] = (uint32_t)(row * (BK * 2) + (((ks * 2 + (lane >> 5)) ^ sw) << 4));
+      const int chunk = F8 ? 4 * (ks / 2) + 2 * (lane >> 5) + ks % 2 : ks * 2 + (lane >> 5);
+      off[ks] = (uint32_t)(row * (BK * 2) + ((chunk ^ sw) << 4));
     }
   }
   __device__ __forceinline__ bf16x8 read(const char* tile, int ks, int blk) const {
@@ -843,14 +864,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
   constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB, KS = BK / 16;
   constexpr bool ACC_F32 = EPI == kEpiAccF32, GATE_UP = EPI == kEpiSwiGLU;
+  // One-byte elements (NT layout only: both operands depth-contiguous).  The tile movers see them
+  // as two-byte elements, two to one: same bytes per row and slice, BK_ELEMS depth values a slice.
+  constexpr bool F8 = is_f8(DT);
+  constexpr int ES = F8 ? 1 : 2, BK_ELEMS = BK * 2 / ES, OUT_DT = DT == kF16 ? kF16 : kBF16;
+  static_assert(!F8 || (LAYOUT == kNT && EPI == kEpiStore && !INDEXED), "fp8 streams in the NT layout, plain store");
   static_assert(!ACC_F32 || LAYOUT == kTN, "the fp32 accumulator is the weight gradient's");
   static_assert(!(GATE_UP || INDEXED) || LAYOUT != kTN, "row indices and gate | up are for the NN and NT layouts");
   static_assert(!GATE_UP || NB % 2 == 0, "a wave needs the gate and the up block of its columns");
   constexpr int BNS = GATE_UP ? BN / 2 : BN;   // output columns per tile, what the schedule counts in
   using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT, INDEXED>, WidthMajor<BM, BK, NT>>;
   using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT, false, GATE_UP>, WidthMajor<BN, BK, NT>>;
-  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK, WAVES_M>, WidthMajorFrag<BM, BK, MB, WAVES_M>>;
-  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK, 1>, WidthMajorFrag<BN, BK, NB, 1>>;
+  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK, WAVES_M, F8>, WidthMajorFrag<BM, BK, MB, WAVES_M>>;
+  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK, 1, F8>, WidthMajorFrag<BN, BK, NB, 1>>;
   constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;   // per lane, per depth slice
   constexpr int QUARTER_LOADS = LOADS_PER_STAGE / 4;
   static_assert(KS == 4 && STAGES == 2, "the step schedule below is written for BK = 64 and two buffers");
@@ -875,7 +901,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // fix-up of the depth pieces stores plain tiles)
   const TailPlan plan = plan_tail<LAYOUT>(
       uniform(sched->tile_start[p.num_groups]) + uniform(sched->runt_start[p.num_groups]),
-      (int)gridDim.x, p, BK, !(GATE_UP || INDEXED));
+      (int)gridDim.x, p, BK_ELEMS, !(GATE_UP || INDEXED));
   const int total_tiles = plan.total;
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
@@ -894,14 +920,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   TileCursor fetch_cur;
   TileInfo fti;
   auto fetch_setup = [&]() {
-    fti = find_tile<LAYOUT, BM, BNS, BK>(sched, p, fetch_t, plan, fetch_cur);
+    fti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, fetch_t, plan, fetch_cur);
     const int depth = fti.depth;
     if constexpr (INDEXED) {
       const int first = fti.g.row0 + fti.m0;
       aload.setup_gather(p.a, p.a_bytes, p.a_rows != nullptr ? p.a_rows + first : nullptr, first, fti.g.k,
                          depth > 0 ? fti.rows_valid : 0, depth);
     } else if constexpr (Cfg::A_DEPTH_MAJOR) {
-      aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * 2, fti.g.k, fti.rows_valid, depth);
+      aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * ES, fti.g.k * ES / 2, fti.rows_valid,
+                  depth * ES / 2);
     } else {
       aload.setup(p.a + fti.g.a_off * 2, fti.g.m, depth, fti.m0, fti.g.m);
     }
@@ -911,8 +938,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     } else if constexpr (GATE_UP) {
       bload.setup_gate_up(p.b + fti.g.b_off * 2, 2 * fti.g.n, depth, fti.n0, fti.g.n);
     } else if constexpr (Cfg::B_DEPTH_MAJOR) {
-      bload.setup(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
-                  fti.valid && depth > 0 ? min(BN, fti.g.n - fti.n0) : 0, depth);
+      bload.setup(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * ES, fti.g.k * ES / 2,
+                  fti.valid && depth > 0 ? min(BN, fti.g.n - fti.n0) : 0, depth * ES / 2);
     } else {
       bload.setup(p.b + fti.g.b_off * 2, fti.g.n, depth, fti.n0, fti.g.n);
     }
@@ -977,7 +1004,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 
   int tile_t = vid;
   TileCursor tile_cur;
-  TileInfo ti = find_tile<LAYOUT, BM, BNS, BK>(sched, p, tile_t, plan, tile_cur);
+  TileInfo ti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, tile_t, plan, tile_cur);
   wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
@@ -1030,20 +1057,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       constexpr int RML = decltype(rml_tag)::value, RUNITS = RML + NB, READS = SETS * RUNITS;
       constexpr int READ_SET = decltype(read_set_tag)::value;
       constexpr int FIRST_LOAD = decltype(first_load_tag)::value, LOADS = decltype(loads_tag)::value;
-      static_for<SLOTS>([&](auto m_tag) {
-        constexpr int m = decltype(m_tag)::value;
+      // fp8: steps 2 s and 2 s + 1 share the 64-deep step s, half of the blocks each, and an
+      // instruction takes the halves 2 s and 2 s + 1 of both fragments
+      constexpr int STEP_SLOTS = F8 ? SLOTS / 2 : SLOTS;
+      static_for<STEP_SLOTS>([&](auto m_tag) {
+        constexpr int mm = decltype(m_tag)::value, m = F8 ? mm + (ks % 2) * STEP_SLOTS : mm;
         // serpentine over the blocks: consecutive MFMAs share one operand, also across rows
         constexpr int j = m / ML, i = (j % 2 == 0) ? m % ML : ML - 1 - m % ML;
         // operands swapped: the result block is held transposed, so a lane owns four
         // consecutive columns of one output row
-        acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
-        constexpr int u0 = READS * m / SLOTS, u1 = READS * (m + 1) / SLOTS;
+        if constexpr (F8) {
+          acc[i][j] = mfma_32x32x64_f8<DT>(fb[ks & ~1][j], fb[ks | 1][j], fa[ks & ~1][i], fa[ks | 1][i], acc[i][j]);
+        } else {
+          acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
+        }
+        constexpr int u0 = READS * mm / STEP_SLOTS, u1 = READS * (mm + 1) / STEP_SLOTS;
         static_for<u1 - u0>([&](auto d) {
           constexpr int u = u0 + decltype(d)::value;
           read_unit(std::integral_constant<int, u % RUNITS>{},
                     std::integral_constant<int, READ_SET + u / RUNITS>{}, rml_tag, src);
         });
-        constexpr int l0 = LOADS * m / SLOTS, l1 = LOADS * (m + 1) / SLOTS;
+        constexpr int l0 = LOADS * mm / STEP_SLOTS, l1 = LOADS * (mm + 1) / STEP_SLOTS;
         static_for<l1 - l0>([&](auto d) {
           fetch_load(std::integral_constant<int, FIRST_LOAD + l0 + decltype(d)::value>{}, fill);
         });
@@ -1120,7 +1154,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[r]) : "a"(acc[i][j][4 * q + r]));
-        return round4<DT>(v[0], v[1], v[2], v[3]);
+        return round4<OUT_DT>(v[0], v[1], v[2], v[3]);
       };
       if constexpr (GATE_UP) {
         // Blocks 2 jp and 2 jp + 1 of a wave hold the gate and the up value of the same 32 output
@@ -1141,7 +1175,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
                 o[r] = gate / (1.0f + __expf(-gate)) * up;
               }
               const int col = ti.n0 + wn * (Cfg::WTN / 2) + jp * 32 + 8 * q + 4 * (lane >> 5);
-              __builtin_amdgcn_raw_buffer_store_b64(round4<DT>(o[0], o[1], o[2], o[3]), rc, at(row_off, col), 0,
+              __builtin_amdgcn_raw_buffer_store_b64(round4<OUT_DT>(o[0], o[1], o[2], o[3]), rc, at(row_off, col), 0,
                                                     kStoreStreaming);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -1251,7 +1285,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     }
     tile_t += G;
     if (tile_t >= total_tiles) break;
-    ti = find_tile<LAYOUT, BM, BNS, BK>(sched, p, tile_t, plan, tile_cur);
+    ti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, tile_t, plan, tile_cur);
   }
   wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
 
@@ -1303,7 +1337,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, old + sum[j][q]), rc, off, 0, 0);
           } else {
             __builtin_amdgcn_raw_buffer_store_b64(
-                round4<DT>(sum[j][q][0], sum[j][q][1], sum[j][q][2], sum[j][q][3]), rc, off, 0, kStoreStreaming);
+                round4<OUT_DT>(sum[j][q][0], sum[j][q][1], sum[j][q][2], sum[j][q][3]), rc, off, 0, kStoreStreaming);
           }
         }
     }

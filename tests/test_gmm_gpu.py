@@ -718,6 +718,42 @@ def test_hip_graph_replay_with_new_device_sizes(ops, oracle):
         check(out, oracle.gmm_loop(a.cpu(), b.cpu(), torch.tensor(new_sizes)), f"replay {new_sizes}")
 
 
+_COLD_CAPTURE = r"""
+import sys, torch
+sys.path.insert(0, sys.argv[1])
+from grouped_gemm import backend
+g = torch.Generator().manual_seed(23)
+a = torch.randn(1500, 256, generator=g).to(torch.bfloat16).cuda()
+b = torch.randn(5, 256, 392, generator=g).to(torch.bfloat16).cuda()
+grad = torch.randn(1500, 392, generator=g).to(torch.bfloat16).cuda()
+sizes = torch.tensor([300] * 5, dtype=torch.int64).cuda()
+out = torch.empty(1500, 392, dtype=torch.bfloat16, device="cuda")
+wgrad = torch.empty(5, 256, 392, dtype=torch.bfloat16, device="cuda")
+torch.cuda.synchronize()
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph):                 # the library's very first calls in this process
+    backend.gmm(a, b, sizes, c=out)
+    backend.gmm(a, grad, sizes, trans_a=True, c=wgrad)
+for new_sizes in ([300] * 5, [1, 2, 3, 4, 1490], [0, 700, 0, 800, 0]):
+    sizes.copy_(torch.tensor(new_sizes, dtype=torch.int64))
+    out.fill_(7.0); wgrad.fill_(7.0)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, backend.gmm(a, b, sizes)), new_sizes
+    assert torch.equal(wgrad, backend.gmm(a, grad, sizes, trans_a=True)), new_sizes
+print("cold capture ok")
+"""
+
+
+def test_hip_graph_capture_of_the_first_call_in_a_process():
+    # No warm-up: the library's first call on the device (set-up of every kernel variant, the
+    # binding's workspace) happens inside the capture; replays with other sizes equal eager calls.
+    import subprocess
+    import sys
+    res = subprocess.run([sys.executable, "-c", _COLD_CAPTURE, ROOT], capture_output=True, text=True, timeout=280)
+    assert res.returncode == 0 and "cold capture ok" in res.stdout, res.stdout[-2000:] + res.stderr[-4000:]
+
+
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_traceable_operator_under_torch_compile(ops, trans_b):
     # one graph, no breaks (fullgraph), forward and both gradients bit-equal to the autograd
@@ -898,6 +934,37 @@ def test_float8_operands(ops, oracle, layout, dtype):
         assert out.dtype == torch.bfloat16
         want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
         check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_float8_streaming_kernel(ops, oracle, dtype):
+    # the NT layout with depths that are multiples of 16 runs on the streaming kernel with the
+    # 32x32x64 fp8 matrix instruction: every count of row blocks, ragged depth and width, the
+    # DeepSeek-style shape shrunk, device- and host-resident sizes
+    cases = [([1, 31, 33, 64, 97, 128, 160, 200, 255, 256, 257, 300, 0, 513], 192, 328),
+             ([300, 0, 17, 1000], 528, 776), ([5] * 70, 272, 136), ([4000], 1024, 512), ([256] * 16, 448, 128)]
+    for idx, (sizes, hin, hout) in enumerate(cases):
+        _announce("fp8 streaming", dtype, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        b = torch.randn(len(sizes), hout, hin, generator=g).to(dtype)
+        out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda() if idx % 2 else bs, trans_b=True)
+        check(out, oracle.gmm_loop(a, b, bs, trans_b=True), f"case {idx}")
+    # exact: one-hot rows against an identity-like weight give the row's value back in its place
+    sizes = [1, 31, 33, 97, 160, 255, 257, 300]
+    bs = torch.tensor(sizes, dtype=torch.int64)
+    t, hin, hout = int(bs.sum()), 256, 384
+    idx = torch.arange(t) % 251
+    rows = torch.zeros(t, hin)
+    rows[torch.arange(t), idx % hin] = (idx % 7 + 1).float()
+    eye = torch.zeros(len(sizes), hout, hin)
+    eye[:, :hin, :] = torch.eye(hin)
+    got = ops.backend.gmm(rows.to(dtype).cuda(), eye.to(dtype).cuda(), bs.cuda(), trans_b=True).float().cpu()
+    want = torch.zeros(t, hout)
+    want[:, :hin] = rows
+    assert torch.equal(got, want)
 
 
 # ------------------------------------------------------------- fused gather / scatter
