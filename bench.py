@@ -194,6 +194,54 @@ def summarize(w, names, layout, ms_per_step, samples, accumulate=False):
     return value, roofline, slowest, kernel_ms
 
 
+def other_paths(steps=5, warmup=2):
+    """The paths past the reference's surface, timed shortly on the forward GEMM of the default
+    workload (8 experts, 32768 rows, 4096 x 14336): fused row gather and scatter, the SwiGLU
+    epilogue (the same b read as gate | up, so half the output width), float16, fp8 (NT layout,
+    e4m3), and hidden sizes that are not multiples of 8 (the general kernels)."""
+    import torch
+    from grouped_gemm import backend
+    from grouped_gemm_amd import workloads
+
+    w = workloads.make(2, device="cuda")
+    sd = w.batch_sizes.cuda()
+    t, flops = w.tokens, w.flops_per_gemm()
+    perm = torch.randperm(t, device="cuda").to(torch.int32)
+    out = torch.empty(t, w.hidden_out, dtype=torch.bfloat16, device="cuda")
+
+    def timed(fn, reps=steps, f=flops):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        return {"ms": round(ms, 4), "TFLOP/s": round(f / (ms * 1e-3) / 1e12, 1)}
+
+    res = {
+        "gather fused (gmm_indexed a_rows)": timed(lambda: backend.gmm_indexed(w.a, w.b, sd, a_rows=perm, c=out)),
+        "scatter fused (gmm_indexed c_rows)": timed(lambda: backend.gmm_indexed(w.a, w.b, sd, c=out, c_rows=perm)),
+        "swiglu epilogue (gmm_swiglu)": timed(lambda: backend.gmm_swiglu(w.a, w.b, sd)),
+    }
+    a16, b16 = w.a.half(), w.b.half()
+    res["float16"] = timed(lambda: backend.gmm(a16, b16, sd, c=out.view(torch.float16)))
+    del a16, b16
+    a8, b8 = w.a.to(torch.float8_e4m3fn), w.b.transpose(1, 2).contiguous().to(torch.float8_e4m3fn)
+    res["float8_e4m3fn, b stored transposed"] = timed(lambda: backend.gmm(a8, b8, sd, trans_b=True, c=out))
+    res["float8_e4m3fn, b stored transposed"]["frac_of_fp8_mfma_peak"] = round(
+        res["float8_e4m3fn, b stored transposed"]["TFLOP/s"] / (2 * PEAK_BF16_TFLOPS), 4)
+    del a8, b8
+    hin, hout = w.hidden_in - 4, w.hidden_out - 4
+    au, bu = w.a[:, :hin].contiguous(), w.b[:, :hin, :hout].contiguous()
+    res[f"hidden sizes {hin} x {hout} (general kernels)"] = timed(lambda: backend.gmm(au, bu, sd), reps=2,
+                                                                 f=2 * t * hin * hout)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -323,6 +371,8 @@ def main():
             }
             del res
         out["other_configs"] = others
+        torch.cuda.empty_cache()
+        out["other_paths"] = other_paths()
     print(json.dumps(out))
 
 

@@ -234,6 +234,9 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   hipStream_t stream = static_cast<hipStream_t>(g.stream);
   const int layout = trans_a ? gg::kTN : (trans_b ? gg::kNT : gg::kNN);
   const int epilogue = out_f32 ? gg::kEpiAccF32 : (swiglu ? gg::kEpiSwiGLU : gg::kEpiStore);
+  // deep groups: the launch is bound by the matrix pipe, and atomic additions to c cost less of
+  // its time than reading, adding and writing; shallow groups: bound by the traffic of c, the reverse
+  const int variant_epilogue = out_f32 && tokens >= (int64_t)kShallowBelow * num_groups ? gg::kEpiAccF32Atomic : epilogue;
   // (the short tile shape exists for two-byte elements, the plain epilogue and rows in place only)
   const bool short_shape = !generic && !swiglu && !indexed && elem_bytes == 2 &&
                            use_short_shape(num_groups, tokens, trans_a);
@@ -242,7 +245,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   const int bn = (generic ? gg::kGenericTileN : (short_shape ? Short::BN : Wide::BN)) / (swiglu ? 2 : 1);
   const gg::VariantOps* variant = nullptr;
   if (!generic) {
-    variant = find_variant(g.dtype, layout, short_shape ? Short::kId : Wide::kId, epilogue, indexed ? 1 : 0);
+    variant = find_variant(g.dtype, layout, short_shape ? Short::kId : Wide::kId, variant_epilogue, indexed ? 1 : 0);
     if (variant == nullptr) return fail(GG_EINVAL, "no kernel for this combination of arguments");
   }
 

@@ -76,6 +76,10 @@ enum : int {
   kEpiStore = 0,    // c in the operands' element type, overwritten
   kEpiAccF32 = 1,   // c in fp32, added to (weight-gradient layout only)
   kEpiSwiGLU = 2,   // b holds gate | up columns; c = silu(a @ gate) * (a @ up), half as wide
+  // kEpiAccF32 with atomic additions instead of read, add, write: faster while the launch is bound
+  // by the matrix pipe (deep groups: 3.35 -> 3.16 ms at 8 x 4096 rows, 4096 x 14336), much slower
+  // when it is bound by the traffic of c itself (256 x 256 rows, 2048 x 7168: 7.0 -> 11.7 ms)
+  kEpiAccF32Atomic = 3,
 };
 
 enum : int {   // debugging switches, for comparing the ways a call can be scheduled
@@ -863,7 +867,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
   constexpr int NT = Cfg::NT, MB = Cfg::MB, NB = Cfg::NB, KS = BK / 16;
-  constexpr bool ACC_F32 = EPI == kEpiAccF32, GATE_UP = EPI == kEpiSwiGLU;
+  constexpr bool ACC_F32 = EPI == kEpiAccF32 || EPI == kEpiAccF32Atomic, GATE_UP = EPI == kEpiSwiGLU;
   // One-byte elements (NT layout only: both operands depth-contiguous).  The tile movers see them
   // as two-byte elements, two to one: same bytes per row and slice, BK_ELEMS depth values a slice.
   constexpr bool F8 = is_f8(DT);
@@ -1182,39 +1186,76 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
           }
         }
       } else if constexpr (ACC_F32) {
-        // c += product in fp32.  The 4 consecutive columns a lane holds are 16 bytes of c:
-        // read them, add, write them back; lanes l and l + 32 cover 32 contiguous bytes of a
-        // row, four such instructions one 128-byte line.  All reads of a 32-row block row are
-        // issued before the first addition: 16 in flight per lane measured faster than a
-        // rolling 8 + 8.
+        if constexpr (EPI == kEpiAccF32Atomic) {
+          // c += product in fp32, by atomic additions that return nothing: the wave fires them and
+          // moves on, where a read-add-write would wait for the reads (every element of c belongs
+          // to one tile, so each gets exactly one addition per call and the result is the same).
+          // One 32 x 32 block at a time goes through the wave's LDS strip, in as the 16-byte pieces
+          // the lanes hold, out as one float per lane, 32 lanes to a row: an instruction then adds
+          // to two complete 128-byte lines.
+          static_assert(Cfg::STAGED_EPILOGUE, "the accumulating epilogue uses the waves' LDS strips");
+          char* strip = smem + Cfg::EPILOGUE_OFFSET + wave * Cfg::EPILOGUE_WAVE_BYTES;
+          constexpr int PITCH = Cfg::EPILOGUE_PITCH;   // 32 floats and 16 bytes of padding
+          const int in_row = lane & 31, in_half = lane >> 5;
 #pragma unroll
-        for (int i = 0; i < ML; ++i) {
-          const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
-          uint32_t off[NB][4];
-          u32x4 old[NB][4];
+          for (int i = 0; i < ML; ++i) {
 #pragma unroll
-          for (int j = 0; j < NB; ++j)
+            for (int j = 0; j < NB; ++j) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
-              off[j][q] = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 4u : kOutOfRange;
-              old[j][q] = __builtin_amdgcn_raw_buffer_load_b128(rc, off[j][q], 0, 0);
-            }
-          __builtin_amdgcn_sched_barrier(0);
+              for (int q = 0; q < 4; ++q) {
+                f32x4 v;
 #pragma unroll
-          for (int j = 0; j < NB; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              f32x4 sum = __builtin_bit_cast(f32x4, old[j][q]);
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                float v;
-                asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
-                sum[r] += v;
+                for (int r = 0; r < 4; ++r)
+                  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v[r]) : "a"(acc[i][j][4 * q + r]));
+                *reinterpret_cast<f32x4*>(strip + in_row * PITCH + (8 * q + 4 * in_half) * 4) = v;
               }
-              __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum), rc, off[j][q], 0, 0);
+              const int col = ti.n0 + wn * Cfg::WTN + j * 32 + (lane & 31);
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const int srow = r * 2 + (lane >> 5);
+                const float v = *reinterpret_cast<const float*>(strip + srow * PITCH + (lane & 31) * 4);
+                const int row = (wm + i * WAVES_M) * 32 + srow;
+                const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 4u : kOutOfRange;
+                __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v, rc, off, 0, 0);
+              }
+              __builtin_amdgcn_sched_barrier(0);
             }
-          __builtin_amdgcn_sched_barrier(0);
+          }
+        } else {
+          // c += product in fp32.  The 4 consecutive columns a lane holds are 16 bytes of c:
+          // read them, add, write them back; lanes l and l + 32 cover 32 contiguous bytes of a
+          // row, four such instructions one 128-byte line.  All reads of a 32-row block row are
+          // issued before the first addition: 16 in flight per lane measured faster than a
+          // rolling 8 + 8.
+#pragma unroll
+          for (int i = 0; i < ML; ++i) {
+            const int row = (wm + i * WAVES_M) * 32 + (lane & 31);
+            uint32_t off[NB][4];
+            u32x4 old[NB][4];
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+                off[j][q] = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * 4u : kOutOfRange;
+                old[j][q] = __builtin_amdgcn_raw_buffer_load_b128(rc, off[j][q], 0, 0);
+              }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                f32x4 sum = __builtin_bit_cast(f32x4, old[j][q]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  float v;
+                  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(acc[i][j][4 * q + r]));
+                  sum[r] += v;
+                }
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sum), rc, off[j][q], 0, 0);
+              }
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
       } else if constexpr (Cfg::STAGED_EPILOGUE) {
         // Through a strip of LDS private to the wave: 32 rows x 64 columns go in as the
