@@ -259,6 +259,9 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   p.b_cols = (int32_t)(swiglu ? 2 * hidden_out : hidden_out);
   p.a_rows = g.a_row_index;
   p.c_rows = g.c_row_index;
+  static_assert(GG_STATUS_NEGATIVE_SIZE == gg::kStatusNegativeSize && GG_STATUS_ROWS_PAST_END == gg::kStatusRowsPastEnd,
+                "the header's status bits are the kernel's");
+  p.status = g.batch_sizes_on_device ? g.size_status : nullptr;
   p.a_bytes = (uint32_t)(indexed_fits ? a_bytes : 0);
   p.c_bytes = (uint32_t)(indexed_fits ? c_bytes : 0);
   p.group_m = band_height(num_groups, tokens, trans_a);

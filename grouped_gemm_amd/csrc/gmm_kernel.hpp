@@ -70,6 +70,12 @@ struct GmmParams {
   const int32_t* c_rows;   // row r of the output goes to row c_rows[r] of c, or nullptr
   uint32_t a_bytes;        // bytes of a and of c in memory, below kOutOfRangeIndexed
   uint32_t c_bytes;
+  int32_t* status;         // device word that collects kStatus* bits about the sizes, or nullptr
+};
+
+enum : int {
+  kStatusNegativeSize = 1,   // a batch size was negative (taken as 0)
+  kStatusRowsPastEnd = 2,    // the sizes sum past `tokens` (the rows past the end were dropped)
 };
 
 enum : int {
@@ -196,8 +202,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
 // Written as assembly on purpose: the compiler then keeps no record of pending writes
 // into LDS, and does not put a full wait for them in front of later LDS reads that touch
 // other buffers of the ring.  The waits that are needed are the explicit wait_vmcnt calls.
-__device__ __forceinline__ void load_to_lds_16(const rsrc_words& rsrc, uint32_t voffset,
+__device__ __forceinline__ void load_to_lds_16(const rsrc_words& rsrc_in, uint32_t voffset,
                                                uint32_t lds_addr) {
+  // (the descriptor is the same in every lane; saying so again here keeps it in scalar registers
+  // even where the compiler has parked it in vector registers for want of scalar ones)
+  rsrc_words rsrc;
+  rsrc[0] = uniform(rsrc_in[0]);
+  rsrc[1] = uniform(rsrc_in[1]);
+  rsrc[2] = uniform(rsrc_in[2]);
+  rsrc[3] = uniform(rsrc_in[3]);
   asm volatile(
       "s_mov_b32 m0, %2\n\t"
       "s_nop 0\n\t"
@@ -306,7 +319,12 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
   const int E = p.num_groups;
   const int per = (E + 63) >> 6;
   const int e0 = lane * per;
-  auto clamp = [&](int64_t v) { return v < 0 ? (int64_t)0 : (v > p.tokens ? p.tokens : v); };
+  int bad = 0;   // kStatus* bits seen by this lane
+  auto clamp = [&](int64_t v) {
+    if (v < 0) bad |= kStatusNegativeSize;
+    if (v > p.tokens) bad |= kStatusRowsPastEnd;
+    return v < 0 ? (int64_t)0 : (v > p.tokens ? p.tokens : v);
+  };
   // rows taken by the groups before this launch's first one
   int64_t base = p.row_base;
   if (p.sizes_dev != nullptr && p.first_group > 0) {
@@ -380,6 +398,14 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
     s->row_start[E] = (int)(run < p.tokens ? run : p.tokens);
     s->tile_start[E] = tincl;
     s->runt_start[E] = rincl;
+    if (run > p.tokens) bad |= kStatusRowsPastEnd;
+  }
+  // What the host would have rejected in host-resident sizes is reported for device-resident
+  // ones: one workgroup ORs what its first wave saw into the caller's status word.
+  if (p.status != nullptr && blockIdx.x == 0) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) bad |= __shfl_xor(bad, d);
+    if (lane == 0 && bad != 0) atomicOr(p.status, bad);
   }
 }
 

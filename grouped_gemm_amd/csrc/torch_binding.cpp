@@ -149,6 +149,19 @@ torch::Tensor Workspace(const torch::Device& device, hipStream_t stream) {
   return it->second;
 }
 
+// One int32 word per device that the kernels OR GG_STATUS_* bits into when device-resident
+// batch_sizes had to be clamped (negative, or summing past the rows of a): what a host-resident
+// size vector would have been rejected for.  Read (and cleared) through size_status().
+torch::Tensor SizeStatusWord(const torch::Device& device) {
+  static std::mutex mu;
+  static std::map<int, torch::Tensor> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find((int)device.index());
+  if (it == cache.end())
+    it = cache.emplace((int)device.index(), torch::zeros({1}, torch::dtype(torch::kInt32).device(device))).first;
+  return it->second;
+}
+
 void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c, const torch::Tensor& batch_sizes,
          bool trans_a, bool trans_b, bool accumulate_f32, int64_t flags, const RowIndices& rows = RowIndices(),
          bool gate_up = false) {
@@ -182,6 +195,7 @@ void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
   g.workspace_bytes = (uint64_t)ws.numel();
   g.flags = (int32_t)flags;
   g.stream = static_cast<void*>(stream);
+  if (sizes.is_cuda()) g.size_status = SizeStatusWord(a.device()).data_ptr<int32_t>();
   const int rc = gg_gmm(&g);
   TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
 }
@@ -239,6 +253,18 @@ void AccumulateWeightGradient(torch::Tensor a, torch::Tensor b, torch::Tensor c,
   Run(a, b, c, batch_sizes, /*trans_a=*/true, /*trans_b=*/false, /*accumulate_f32=*/true, /*flags=*/0);
 }
 
+// GG_STATUS_* bits collected on `device` since the last call of this function (waits for the
+// device): 0 unless device-resident batch_sizes had to be clamped.
+int64_t SizeStatus(torch::Device device) {
+  TORCH_CHECK(device.is_cuda(), "grouped_gemm: size_status is kept per GPU");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(device);
+  if (!device.has_index()) device = torch::Device(device.type(), c10::hip::current_device());
+  torch::Tensor word = SizeStatusWord(device);
+  const int64_t bits = word.item<int32_t>();
+  if (bits != 0) word.zero_();
+  return bits;
+}
+
 // The on-device scheduler's view of the groups, as an int64 tensor
 // (num_experts, GG_SCHED_COLS) on `device`; see gg_debug_schedule.
 torch::Tensor DebugSchedule(torch::Tensor batch_sizes, int64_t tokens, int64_t hidden_in,
@@ -270,6 +296,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gmm_swiglu", &GroupedGemmSwiGLU, "silu(a @ gate) * (a @ up) with b = [gate | up].", py::arg("a"),
         py::arg("b"), py::arg("c"), py::arg("batch_sizes"), py::arg("trans_b"), py::arg("a_rows") = py::none(),
         py::arg("c_rows") = py::none());
+  m.def("size_status", &SizeStatus,
+        "Bits collected since the last call: 1 a device-resident batch size was negative, 2 they summed past the "
+        "rows of a (both clamped by the kernel).");
+  m.attr("status_negative_size") = GG_STATUS_NEGATIVE_SIZE;
+  m.attr("status_rows_past_end") = GG_STATUS_ROWS_PAST_END;
   m.def("gmm_with_flags", &GroupedGemmWithFlags, "gmm with GG_FLAG_* bits (testing).");
   m.attr("flag_whole_tiles") = GG_FLAG_WHOLE_TILES;
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,

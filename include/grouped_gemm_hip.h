@@ -43,6 +43,10 @@ extern "C" {
 #define GG_DTYPE_F8E4M3 2   /* OCP e4m3 (torch.float8_e4m3fn) in a and b, bf16 in c */
 #define GG_DTYPE_F8E5M2 3   /* OCP e5m2 (torch.float8_e5m2) in a and b, bf16 in c */
 
+/* bits a launch ORs into *gg_gmm_args.size_status */
+#define GG_STATUS_NEGATIVE_SIZE 1   /* a device-resident batch size was negative (taken as 0) */
+#define GG_STATUS_ROWS_PAST_END 2   /* device-resident sizes sum past `tokens` (rows past the end dropped) */
+
 /* gg_gmm_args.epilogue */
 #define GG_EPILOGUE_NONE 0
 #define GG_EPILOGUE_SWIGLU 1   /* b holds gate | up columns; c = silu(a @ gate) * (a @ up) */
@@ -144,6 +148,11 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  *                 With two-byte elements, aligned operands and a and c below 4 GiB the NN and NT
  *                 layouts run indexed on the streaming kernels; otherwise, and with trans_a, on
  *                 the general ones.
+ *   size_status   int32 word on the device, or NULL.  Host-resident batch_sizes that are negative
+ *                 or sum past `tokens` are rejected; device-resident ones cannot be (the host
+ *                 never reads them) and are clamped instead.  With a status word the kernel ORs
+ *                 GG_STATUS_* bits into it when it had to clamp, for the caller to read whenever
+ *                 it next synchronises.  Never cleared by the library.
  *   epilogue      GG_EPILOGUE_SWIGLU (not with trans_a or accumulate_f32): b holds two matrices
  *                 per group side by side, gate and up: (num_groups, hidden_in, 2 * hidden_out), or
  *                 (num_groups, 2 * hidden_out, hidden_in) with trans_b, gate first.  c (tokens,
@@ -191,6 +200,7 @@ typedef struct gg_gmm_args {
   int64_t c_num_rows;
   int32_t epilogue;
   int32_t reserved1;
+  int32_t* size_status;
 } gg_gmm_args;
 
 int gg_gmm(const gg_gmm_args* args);

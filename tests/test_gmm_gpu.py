@@ -544,7 +544,7 @@ class GmmArgs(ctypes.Structure):
                 ("flags", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("stream", ctypes.c_void_p),
                 ("a_row_index", ctypes.c_void_p), ("b_row_index", ctypes.c_void_p), ("c_row_index", ctypes.c_void_p),
                 ("a_num_rows", ctypes.c_int64), ("c_num_rows", ctypes.c_int64),
-                ("epilogue", ctypes.c_int32), ("reserved1", ctypes.c_int32)]
+                ("epilogue", ctypes.c_int32), ("reserved1", ctypes.c_int32), ("size_status", ctypes.c_void_p)]
 
 
 def _gmm_args(lib, a, b, c, sizes, on_device, tokens, hin, hout, trans_a, trans_b, flags=0, workspace=None,
@@ -1267,6 +1267,29 @@ def test_output_fully_overwritten_and_tail_rows_untouched(ops, oracle):
     assert not torch.isnan(c[:340]).any()
     assert torch.isnan(c[340:]).all()
     check(c[:340], oracle.gmm_loop(a.cpu(), b.cpu(), sizes)[:340], "forward")
+
+
+def test_clamped_device_sizes_are_reported(ops, oracle):
+    # host-resident sizes that are negative or sum past the rows of a raise; device-resident ones
+    # are clamped by the kernel (it must not follow them) and the fact is left in a status word
+    be = ops.backend.backend
+    dev = torch.device("cuda", torch.cuda.current_device())
+    be.size_status(dev)                                                   # clear
+    g = torch.Generator().manual_seed(13)
+    a = torch.randn(150, 64, generator=g).to(torch.bfloat16).cuda()
+    b = torch.randn(3, 64, 72, generator=g).to(torch.bfloat16).cuda()
+    ops.backend.gmm(a, b, torch.tensor([100, 30, 20]).cuda())
+    assert be.size_status(dev) == 0
+    for sizes, bits, used in [([100, 100, 100], be.status_rows_past_end, [100, 50, 0]),
+                              ([-5, 100, 50], be.status_negative_size, [0, 100, 50]),
+                              ([-1, 149, 7], be.status_negative_size | be.status_rows_past_end, [0, 149, 1])]:
+        with pytest.raises(RuntimeError):
+            ops.backend.gmm(a, b, torch.tensor(sizes))
+        out = ops.backend.gmm(a, b, torch.tensor(sizes).cuda())
+        assert be.size_status(dev) == bits, sizes
+        assert be.size_status(dev) == 0                                   # reading clears
+        rows = sum(used)
+        check(out[:rows], oracle.gmm_loop(a.cpu(), b.cpu(), torch.tensor(used))[:rows], f"clamped {sizes}")
 
 
 def test_all_experts_empty(ops):
