@@ -117,9 +117,8 @@ struct TailPlan {
   int total;        // indices to hand out: main_tiles + rest * pieces
   bool by_depth;
 };
-template <int LAYOUT>
-__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmParams& p, int bk,
-                                              bool depth_pieces_allowed = true) {
+template <int LAYOUT, bool DEPTH_PIECES_ALLOWED = true>
+__device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmParams& p, int bk) {
   TailPlan t;
   const int rest = tiles % grid;
   t.pieces = 1;
@@ -127,7 +126,7 @@ __device__ __forceinline__ TailPlan plan_tail(int tiles, int grid, const GmmPara
   if (rest > 0 && 2 * rest <= grid && !(p.flags & kFlagWholeTiles)) {
     int cand = grid / rest;
     cand = cand > kMaxDepthPieces ? kMaxDepthPieces : cand;
-    if (p.ws_slots > 0 && depth_pieces_allowed && !(p.flags & kFlagRowPieces)) {
+    if (DEPTH_PIECES_ALLOWED && p.ws_slots > 0 && !(p.flags & kFlagRowPieces)) {
       if (rest * cand > p.ws_slots) cand = p.ws_slots / rest;
       cand = cand >= 4 ? 4 : cand;
       if (LAYOUT != kTN) {   // the depth is the same for every tile: keep the pieces worth their fix-up
@@ -929,9 +928,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 
   // (a tile that is combined or scattered on its way out is never cut along the depth: the
   // fix-up of the depth pieces stores plain tiles)
-  const TailPlan plan = plan_tail<LAYOUT>(
+  constexpr bool DEPTH_PIECES = !(GATE_UP || INDEXED);
+  TailPlan plan = plan_tail<LAYOUT, DEPTH_PIECES>(
       uniform(sched->tile_start[p.num_groups]) + uniform(sched->runt_start[p.num_groups]),
-      (int)gridDim.x, p, BK_ELEMS, !(GATE_UP || INDEXED));
+      (int)gridDim.x, p, BK_ELEMS);
+  if constexpr (!DEPTH_PIECES) plan.by_depth = false;   // (known at compile time: no depth-piece code is kept)
   const int total_tiles = plan.total;
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
@@ -1135,7 +1136,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     // A depth piece of a tile of the last round: park the partial tile in the workspace and
     // count the arrival.  The piece that arrives last adds the partial tiles up and stores the
     // sum, after the tile loop (fix_up below), where no accumulator is live any more.
-    if (ti.pieces > 1) {
+    if (DEPTH_PIECES && ti.pieces > 1) {
       float* mine = partial_slot(ti.piece);
 #pragma unroll
       for (int i = 0; i < ML; ++i)
@@ -1361,7 +1362,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // in piece order, two per step (their count is even), whichever piece does the adding, so the
   // result does not depend on timing.  One block row of 32 rows at a time: NB * 4 groups of 16
   // bytes per lane and piece.
-  if (fix_pending) {
+  if (DEPTH_PIECES && fix_pending) {
     __threadfence();   // the other pieces' partial tiles are visible to this workgroup
     if (threadIdx.x == 0) reinterpret_cast<int*>(p.workspace)[ti.rank] = 0;   // leave the counters as they were found
     constexpr int CE = ACC_F32 ? 4 : 2;   // bytes per element of c

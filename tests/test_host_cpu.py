@@ -134,8 +134,8 @@ def _declared_functions():
 
 def test_c_abi_exports_every_declared_symbol():
     names = _declared_functions()
-    assert {"gg_gmm_bf16", "gg_gmm", "gg_init", "gg_gmm_bf16_acc_f32", "gg_debug_schedule", "gg_last_error",
-            "gg_version", "gg_tile_shape"} <= set(names)
+    assert {"gg_gmm_bf16", "gg_gmm", "gg_gmm_no_alloc", "gg_init", "gg_gmm_bf16_acc_f32", "gg_debug_schedule",
+            "gg_last_error", "gg_version", "gg_tile_shape"} <= set(names)
     lib = ctypes.CDLL(HIP_LIB)
     for n in names:
         assert hasattr(lib, n), n
@@ -172,6 +172,70 @@ def test_c_abi_argument_errors_need_no_device():
     assert bm.value == 128          # few rows per group: the shorter tile
     assert bm.value > 0 and bn.value > 0 and bk.value > 0
     assert lib.gg_version() >= 100
+
+
+def test_validate_element_types():
+    # past the reference (bfloat16 only, grouped_gemm.cu:492, 505-506): float16 for all three
+    # tensors alike; float8 operands with a bfloat16 output
+    _validate(a_t=torch.zeros(8, 16, dtype=torch.float16), b_t=torch.zeros(2, 16, 24, dtype=torch.float16),
+              c_t=torch.zeros(8, 24, dtype=torch.float16))
+    for f8 in (torch.float8_e4m3fn, torch.float8_e5m2):
+        _validate(a_t=torch.zeros(8, 16, dtype=f8), b_t=torch.zeros(2, 16, 24, dtype=f8))     # c bfloat16
+        with pytest.raises(RuntimeError):
+            _validate(a_t=torch.zeros(8, 16, dtype=f8), b_t=torch.zeros(2, 16, 24, dtype=f8),
+                      c_t=torch.zeros(8, 24, dtype=f8))
+    with pytest.raises(RuntimeError):
+        _validate(a_t=torch.zeros(8, 16, dtype=torch.float16), b_t=torch.zeros(2, 16, 24, dtype=torch.float16))
+    with pytest.raises(RuntimeError):
+        _validate(a_t=torch.zeros(8, 16, dtype=torch.float8_e4m3fn), b_t=torch.zeros(2, 16, 24, dtype=torch.float8_e5m2))
+
+
+class _Args(ctypes.Structure):
+    """gg_gmm_args of include/grouped_gemm_hip.h."""
+    _fields_ = [("struct_bytes", ctypes.c_uint32), ("dtype", ctypes.c_int32),
+                ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p),
+                ("batch_sizes", ctypes.c_void_p), ("batch_sizes_on_device", ctypes.c_int32),
+                ("trans_a", ctypes.c_int32), ("trans_b", ctypes.c_int32), ("accumulate_f32", ctypes.c_int32),
+                ("num_groups", ctypes.c_int64), ("tokens", ctypes.c_int64),
+                ("hidden_in", ctypes.c_int64), ("hidden_out", ctypes.c_int64),
+                ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_uint64),
+                ("flags", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("stream", ctypes.c_void_p),
+                ("a_row_index", ctypes.c_void_p), ("b_row_index", ctypes.c_void_p), ("c_row_index", ctypes.c_void_p),
+                ("a_num_rows", ctypes.c_int64), ("c_num_rows", ctypes.c_int64),
+                ("epilogue", ctypes.c_int32), ("reserved1", ctypes.c_int32), ("size_status", ctypes.c_void_p)]
+
+
+def test_general_entry_point_argument_errors_need_no_device():
+    lib = ctypes.CDLL(HIP_LIB)
+    lib.gg_last_error.restype = ctypes.c_char_p
+    lib.gg_gmm.argtypes = [ctypes.c_void_p]
+    sizes = (ctypes.c_int64 * 2)(3, 5)
+
+    def call(**kw):
+        g = _Args()
+        g.struct_bytes = ctypes.sizeof(_Args)
+        g.a, g.b, g.c = 4096, 8192, 12288            # never dereferenced: every case fails before the device
+        g.batch_sizes = ctypes.addressof(sizes)
+        g.num_groups, g.tokens, g.hidden_in, g.hidden_out = 2, 8, 16, 24
+        for k, v in kw.items():
+            setattr(g, k, v)
+        return lib.gg_gmm(ctypes.byref(g)), lib.gg_last_error()
+
+    assert call(struct_bytes=8)[0] == -1
+    assert lib.gg_gmm(None) == -1
+    assert call(dtype=9) == (-1, b"dtype must be one of GG_DTYPE_*")
+    assert call(epilogue=7)[0] == -1
+    rc, msg = call(epilogue=1, trans_a=1)
+    assert rc == -1 and b"SwiGLU" in msg
+    rc, msg = call(accumulate_f32=1)
+    assert rc == -1 and b"trans_a" in msg
+    rc, msg = call(trans_a=1, c_row_index=64)
+    assert rc == -1 and b"c_row_index" in msg
+    rc, msg = call(b_row_index=64)
+    assert rc == -1 and b"b_row_index" in msg
+    assert call(a_num_rows=-1)[0] == -1
+    rc, msg = call(c=12288 + 1)
+    assert rc == -2 and b"element size" in msg
 
 
 # ----------------------------------------------------------------- workloads
