@@ -32,11 +32,20 @@ PEAK_HBM_GBPS = 8000.0
 # runs of this file (FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by a 1 GiB device copy, both in
 # KiB).  Profiled once, not in this run: `source` names the summary under profiles/ that holds the
 # figures, the commands and the revision of the kernel they were taken on.
-_TRAFFIC_SOURCE = "profiles/gmm_kernel_mixtral_w1_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, profiled once)"
+_TRAFFIC_SOURCE = ("profiles/gmm_kernel_mixtral_w1_hbm_traffic.md and profiles/gmm_kernel_configs_3_4_5_stats_and_traffic.md "
+                   "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel revision with runt rows last and depth "
+                   "pieces; profiled once, not in this run)")
+
+
+def _traffic(fetch_kib, write_kib):
+    return {"bytes": (fetch_kib * 2.0 + write_kib) * 1024, "source": _TRAFFIC_SOURCE}
+
+
 MEASURED_TRAFFIC = {
-    2: {"fwd": {"bytes": (4458000 * 2.0 + 917600) * 1024, "source": _TRAFFIC_SOURCE},
-        "agrad": {"bytes": (3812000 * 2.0 + 262144) * 1024, "source": _TRAFFIC_SOURCE},
-        "bgrad": {"bytes": (2755000 * 2.0 + 917500) * 1024, "source": _TRAFFIC_SOURCE}},
+    2: {"fwd": _traffic(4088250, 917549), "agrad": _traffic(3325500, 290120), "bgrad": _traffic(2753350, 917545)},
+    3: {"fwd": _traffic(435980, 135184)},
+    4: {"bgrad": _traffic(2752720, 917516)},
+    5: {"fwd": _traffic(4359720, 262158), "agrad": _traffic(5455520, 917508), "bgrad": _traffic(1851630, 7342490)},
 }
 
 
