@@ -69,10 +69,12 @@ class GroupedGemmGather(torch.autograd.Function):
             xgrad.index_add_(0, row_index.long(), sorted_grad.float())
             xgrad = xgrad.to(x.dtype)
         if ctx.needs_input_grad[1]:
-            if ctx.trans_b:
-                wgrad = backend.gmm_indexed(grad, x, batch_sizes, trans_a=True, b_rows=row_index)
-            else:
-                wgrad = backend.gmm_indexed(x, grad, batch_sizes, trans_a=True, a_rows=row_index)
+            # The weight-gradient layout takes row indices on the general kernels only, which are
+            # several times slower than the streaming ones: one explicit gather and the streaming
+            # kernel is the faster way to the same result.
+            sorted_x = x.index_select(0, row_index.long())
+            lhs, rhs = (grad, sorted_x) if ctx.trans_b else (sorted_x, grad)
+            wgrad = backend.gmm(lhs, rhs, batch_sizes, trans_a=True)
         return xgrad, wgrad, None, None, None
 
 
@@ -96,10 +98,10 @@ class GroupedGemmScatter(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             agrad = backend.gmm_indexed(grad, w, batch_sizes, trans_b=not ctx.trans_b, a_rows=row_index)
         if ctx.needs_input_grad[1]:
-            if ctx.trans_b:
-                wgrad = backend.gmm_indexed(grad, a, batch_sizes, trans_a=True, a_rows=row_index)
-            else:
-                wgrad = backend.gmm_indexed(a, grad, batch_sizes, trans_a=True, b_rows=row_index)
+            # (as in GroupedGemmGather: an explicit gather, then the streaming weight-gradient kernel)
+            sorted_grad = grad.index_select(0, row_index.long())
+            lhs, rhs = (sorted_grad, a) if ctx.trans_b else (a, sorted_grad)
+            wgrad = backend.gmm(lhs, rhs, batch_sizes, trans_a=True)
         return agrad, wgrad, None, None, None
 
 
