@@ -3,10 +3,16 @@
   libgrouped_gemm_hip.so            HIP kernels + C ABI (hipcc, gfx950 only)
   grouped_gemm_backend.<abi>.so     PyTorch-ROCm binding (g++, links the first)
 
-Usage: python grouped_gemm_amd/build.py [--force]
+Usage: python grouped_gemm_amd/build.py [--force] [--diagnostic no_loads|no_mfma]
 hipcc cross-compiles gfx950 without a GPU, so this runs anywhere the ROCm toolchain
 and PyTorch-ROCm are installed.  The kernel variants (csrc/gmm_variants.def) are compiled as
 separate translation units, several at a time; objects are kept under grouped_gemm_amd/build/.
+
+--diagnostic NAME builds a second copy of the kernel library with GG_DIAGNOSTIC_<NAME> defined
+(csrc/gmm_kernel.hpp: the kernels without their operand loads, or without their matrix
+instructions; wrong results, for timing only) into grouped_gemm_amd/diagnostic/NAME/.  Nothing
+loads it unless that directory is put first on LD_LIBRARY_PATH, e.g.
+LD_LIBRARY_PATH=grouped_gemm_amd/diagnostic/no_mfma python bench.py --config 5 --no-cpu-baseline
 """
 import os
 import re
@@ -58,19 +64,26 @@ def variant_indices():
     return [int(m) for m in re.findall(r"^GG_VARIANT\((\d+),", text, flags=re.M)]
 
 
-def build_hip(force=False, jobs=None):
+def build_hip(force=False, jobs=None, diagnostic=None):
     headers = [os.path.join(CSRC, f) for f in ("gmm_kernel.hpp", "gmm_generic.hpp", "gmm_variants.hpp",
                                                "gmm_variants.def")]
     headers.append(os.path.join(ROOT, "include", "grouped_gemm_hip.h"))
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    os.makedirs(OBJ_DIR, exist_ok=True)
-    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(OBJ_DIR, "gmm_api.o"), [])]
+    obj_dir, hip_lib, extra = OBJ_DIR, HIP_LIB, []
+    if diagnostic:
+        if diagnostic not in ("no_loads", "no_mfma"):
+            raise ValueError("--diagnostic takes no_loads or no_mfma")
+        obj_dir = os.path.join(HERE, "diagnostic", diagnostic)
+        hip_lib = os.path.join(obj_dir, os.path.basename(HIP_LIB))
+        extra = ["-DGG_DIAGNOSTIC_" + diagnostic.upper()]
+    os.makedirs(obj_dir, exist_ok=True)
+    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(obj_dir, "gmm_api.o"), extra)]
     for i in variant_indices():
-        units.append((os.path.join(CSRC, "gmm_variant.hip"), os.path.join(OBJ_DIR, f"gmm_variant_{i}.o"),
-                      [f"-DGG_VARIANT_INDEX={i}"]))
+        units.append((os.path.join(CSRC, "gmm_variant.hip"), os.path.join(obj_dir, f"gmm_variant_{i}.o"),
+                      extra + [f"-DGG_VARIANT_INDEX={i}"]))
     for dt in range(4):   # gmm_generic.hpp, one translation unit per element type
-        units.append((os.path.join(CSRC, "gmm_generic_variant.hip"), os.path.join(OBJ_DIR, f"gmm_generic_{dt}.o"),
-                      [f"-DGG_GENERIC_DT={dt}"]))
+        units.append((os.path.join(CSRC, "gmm_generic_variant.hip"), os.path.join(obj_dir, f"gmm_generic_{dt}.o"),
+                      extra + [f"-DGG_GENERIC_DT={dt}"]))
     todo = [u for u in units if force or not _newer(u[1], [u[0]] + headers)]
     jobs = jobs or min(len(todo) or 1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1)))
     if todo:
@@ -78,9 +91,9 @@ def build_hip(force=False, jobs=None):
         with ThreadPoolExecutor(max_workers=jobs) as pool:
             list(pool.map(lambda u: _run([hipcc] + HIPCC_FLAGS + u[2] + ["-c", u[0], "-o", u[1]], quiet=True), todo))
     objects = [u[1] for u in units]
-    if todo or not _newer(HIP_LIB, objects):
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", HIP_LIB])
-    return HIP_LIB
+    if todo or not _newer(hip_lib, objects):
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objects + ["-o", hip_lib])
+    return hip_lib
 
 
 def build_binding(force=False):
@@ -116,4 +129,7 @@ def build_all(force=False):
 
 
 if __name__ == "__main__":
-    build_all(force="--force" in sys.argv)
+    if "--diagnostic" in sys.argv:
+        print(build_hip(force="--force" in sys.argv, diagnostic=sys.argv[sys.argv.index("--diagnostic") + 1]))
+    else:
+        build_all(force="--force" in sys.argv)

@@ -881,6 +881,21 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   return ti;
 }
 
+// Diagnostic builds (build.py --diagnostic no_loads | no_mfma), for timing only, results are
+// wrong: GG_DIAGNOSTIC_NO_LOADS leaves out the loads of the operand tiles (what remains: matrix
+// instructions, LDS reads, barriers, epilogue), GG_DIAGNOSTIC_NO_MFMA all but one matrix
+// instruction per step (what remains: the fetch pipeline, the LDS reads and the epilogue).
+#ifdef GG_DIAGNOSTIC_NO_LOADS
+constexpr bool kDiagnosticNoLoads = true;
+#else
+constexpr bool kDiagnosticNoLoads = false;
+#endif
+#ifdef GG_DIAGNOSTIC_NO_MFMA
+constexpr bool kDiagnosticNoMfma = true;
+#else
+constexpr bool kDiagnosticNoMfma = false;
+#endif
+
 // DT: element type of a and b (and of c unless it is the fp32 accumulator).
 // EPI: what happens to a finished tile (kEpi*): stored in the element type; added to an fp32 c
 // (gradient accumulation, weight-gradient layout); or, with gate | up columns in b, combined to
@@ -987,7 +1002,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   auto fetch_load = [&](auto j_tag, int buf) {
     constexpr int J = decltype(j_tag)::value;
     const char* st = smem + buf * Cfg::STAGE_BYTES;
-    if constexpr (J < ALoad::NI) {
+    if constexpr (kDiagnosticNoLoads) {
+    } else if constexpr (J < ALoad::NI) {
       aload.template load<J>(a_slice, st, wave);
     } else {
       bload.template load<J - ALoad::NI>(b_slice, st + Cfg::A_BYTES, wave);
@@ -1097,10 +1113,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
         constexpr int j = m / ML, i = (j % 2 == 0) ? m % ML : ML - 1 - m % ML;
         // operands swapped: the result block is held transposed, so a lane owns four
         // consecutive columns of one output row
-        if constexpr (F8) {
-          acc[i][j] = mfma_32x32x64_f8<DT>(fb[ks & ~1][j], fb[ks | 1][j], fa[ks & ~1][i], fa[ks | 1][i], acc[i][j]);
-        } else {
-          acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
+        if constexpr (!kDiagnosticNoMfma || mm == 0) {
+          if constexpr (F8) {
+            acc[i][j] = mfma_32x32x64_f8<DT>(fb[ks & ~1][j], fb[ks | 1][j], fa[ks & ~1][i], fa[ks | 1][i], acc[i][j]);
+          } else {
+            acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
+          }
         }
         constexpr int u0 = READS * mm / STEP_SLOTS, u1 = READS * (mm + 1) / STEP_SLOTS;
         static_for<u1 - u0>([&](auto d) {
