@@ -329,6 +329,21 @@ def main():
     }
     if args.flags:
         out["config"]["diagnostic_flags"] = args.flags
+    # What the chip sustains on the matrix instruction alone (operands in registers, no memory
+    # traffic), right after the timed region: on operands with the bit statistics of this data the
+    # power limit lowers the clock, on zeros it does not.  The first figure is the ceiling of any
+    # bf16 GEMM on this device and data.
+    from grouped_gemm import backend as _backend
+    dev = torch.device("cuda", 0)
+    pipe_random = _backend.backend.mfma_rate(dev, False, 10)
+    pipe_zeros = _backend.backend.mfma_rate(dev, True, 10)
+    out["matrix_pipe_alone"] = {
+        "what": "v_mfma_f32_32x32x16_bf16 on register operands, 256 workgroups of 4 waves, 10 launches of about 2.5 ms",
+        "random_operands_TFLOP/s": round(pipe_random, 1),
+        "zero_operands_TFLOP/s": round(pipe_zeros, 1),
+        "random_operands_frac_of_peak": round(pipe_random / PEAK_BF16_TFLOPS, 4),
+        "value_over_random_operands_rate": round(value / pipe_random, 4),
+    }
     if args.vendor_loop:
         # the NN launch of this workload: forward, or the input gradient when b is stored transposed
         which = "agrad" if w.trans_b else "fwd"

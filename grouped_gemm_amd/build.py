@@ -77,7 +77,8 @@ def build_hip(force=False, jobs=None, diagnostic=None):
         hip_lib = os.path.join(obj_dir, os.path.basename(HIP_LIB))
         extra = ["-DGG_DIAGNOSTIC_" + diagnostic.upper()]
     os.makedirs(obj_dir, exist_ok=True)
-    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(obj_dir, "gmm_api.o"), extra)]
+    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(obj_dir, "gmm_api.o"), extra),
+             (os.path.join(CSRC, "gmm_probe.hip"), os.path.join(obj_dir, "gmm_probe.o"), extra)]
     for i in variant_indices():
         units.append((os.path.join(CSRC, "gmm_variant.hip"), os.path.join(obj_dir, f"gmm_variant_{i}.o"),
                       extra + [f"-DGG_VARIANT_INDEX={i}"]))

@@ -451,4 +451,16 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   return dispatch_dump(short_shape, layout, p, hs, stream);
 }
 
+int gg_debug_mfma_rate(int zero_operands, int launches, void* stream, float* tflops) {
+  if (tflops == nullptr) return fail(GG_EINVAL, "tflops is null");
+  if (launches < 1 || launches > 1000) return fail(GG_EINVAL, "launches must be 1 .. 1000");
+  DeviceInfo info;
+  const int rc = device_info(&info);
+  if (rc != GG_OK) return rc;
+  // (the kernel never writes through this pointer: the static scratch array is merely a valid one)
+  GG_HIP(gg::run_mfma_probe(info.cus, zero_operands != 0, launches, reinterpret_cast<float*>(info.scratch),
+                            static_cast<hipStream_t>(stream), tflops));
+  return GG_OK;
+}
+
 }  // extern "C"

@@ -284,6 +284,19 @@ torch::Tensor DebugSchedule(torch::Tensor batch_sizes, int64_t tokens, int64_t h
   return out;
 }
 
+// TFLOP/s the device sustains on the bf16 matrix instruction alone, operands in registers
+// (see gg_debug_mfma_rate); waits for the device.
+double MfmaRate(torch::Device device, bool zero_operands, int64_t launches) {
+  TORCH_CHECK(device.is_cuda(), "grouped_gemm: the probe runs on a GPU");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(device);
+  if (!device.has_index()) device = torch::Device(device.type(), c10::hip::current_device());
+  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index()).stream();
+  float tflops = 0.0f;
+  const int rc = gg_debug_mfma_rate(zero_operands ? 1 : 0, (int)launches, static_cast<void*>(stream), &tflops);
+  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
+  return tflops;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gmm", &GroupedGemm, "Grouped GEMM.");
   m.def("validate",
@@ -306,6 +319,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,
         "c (fp32) += per expert a_e^T @ b_e.");
   m.def("debug_schedule", &DebugSchedule, "Per-group table derived by the on-device scheduler.");
+  m.def("mfma_rate", &MfmaRate, "TFLOP/s of the bf16 matrix instruction alone, operands in registers.",
+        py::arg("device"), py::arg("zero_operands") = false, py::arg("launches") = 5);
   m.attr("max_groups_per_launch") = GG_MAX_GROUPS_PER_LAUNCH;
   m.attr("sched_cols") = GG_SCHED_COLS;
 }

@@ -236,6 +236,16 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device,
                       int64_t hidden_out, int trans_a, int trans_b, int64_t* table_out,
                       void* stream);
 
+/*
+ * A probe, no counterpart in the reference: the rate (TFLOP/s, through `tflops`) at which the
+ * device sustains the bf16 matrix instruction the kernels are built on, with operands in
+ * registers and no memory traffic; on operands with the bit statistics of randn * 0.02 data
+ * (zero_operands = 0) or on zeros.  The first is the ceiling the device's power limit sets for any
+ * bf16 GEMM on such data; benchmarks print it next to the GEMM's rate.  Runs `launches` + 1
+ * launches of about 2 ms on `stream` and waits for them.
+ */
+int gg_debug_mfma_rate(int zero_operands, int launches, void* stream, float* tflops);
+
 /* Output tile (rows, columns) and depth slice the kernel uses for a call with these arguments
  * (calls whose groups average few rows get a shorter tile); for reports and for checking the
  * tile counts of gg_debug_schedule. */

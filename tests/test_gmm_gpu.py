@@ -1381,3 +1381,15 @@ def test_runs_on_the_current_stream(ops, oracle):
         out = ops.backend.gmm(a2, b, sizes.cuda())
     s.synchronize()
     check(out / 2, oracle.gmm_loop(a.cpu(), b.cpu(), sizes), "forward")
+
+
+def test_matrix_pipe_probe(ops):
+    """gg_debug_mfma_rate: a rate between nothing and the published peak, and no slower on zeros
+    than on operands whose bits toggle."""
+    dev = torch.device("cuda", 0)
+    rate_random = ops.backend.backend.mfma_rate(dev, False, 2)
+    rate_zeros = ops.backend.backend.mfma_rate(dev, True, 2)
+    assert 100.0 < rate_random < 2600.0 and 100.0 < rate_zeros < 2600.0, (rate_random, rate_zeros)
+    assert rate_zeros > 0.9 * rate_random, (rate_random, rate_zeros)
+    with pytest.raises(RuntimeError):
+        ops.backend.backend.mfma_rate(dev, False, 0)
