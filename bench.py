@@ -206,8 +206,8 @@ def summarize(w, names, layout, ms_per_step, samples, accumulate=False):
 def other_paths(steps=5, warmup=2):
     """The paths past the reference's surface, timed shortly on the forward GEMM of the default
     workload (8 experts, 32768 rows, 4096 x 14336): fused row gather and scatter, the SwiGLU
-    epilogue (the same b read as gate | up, so half the output width), float16, fp8 (NT layout,
-    e4m3), and hidden sizes that are not multiples of 8 (the general kernels)."""
+    epilogue (the same b read as gate | up, so half the output width), float16, fp8 (e4m3, b as
+    stored and b stored transposed, and the weight gradient), and hidden sizes that are not multiples of 8 (the general kernels)."""
     import torch
     from grouped_gemm import backend
     from grouped_gemm_amd import workloads
@@ -241,9 +241,16 @@ def other_paths(steps=5, warmup=2):
     del a16, b16
     a8, b8 = w.a.to(torch.float8_e4m3fn), w.b.transpose(1, 2).contiguous().to(torch.float8_e4m3fn)
     res["float8_e4m3fn, b stored transposed"] = timed(lambda: backend.gmm(a8, b8, sd, trans_b=True, c=out))
-    res["float8_e4m3fn, b stored transposed"]["frac_of_fp8_mfma_peak"] = round(
-        res["float8_e4m3fn, b stored transposed"]["TFLOP/s"] / (2 * PEAK_BF16_TFLOPS), 4)
-    del a8, b8
+    del b8
+    b8 = w.b.to(torch.float8_e4m3fn)
+    res["float8_e4m3fn"] = timed(lambda: backend.gmm(a8, b8, sd, c=out))
+    del b8
+    g8 = w.grad.to(torch.float8_e4m3fn)
+    wgrad = torch.empty_like(w.b)
+    res["float8_e4m3fn, weight gradient (trans_a)"] = timed(lambda: backend.gmm(a8, g8, sd, trans_a=True, c=wgrad))
+    for key in ("float8_e4m3fn, b stored transposed", "float8_e4m3fn", "float8_e4m3fn, weight gradient (trans_a)"):
+        res[key]["frac_of_fp8_mfma_peak"] = round(res[key]["TFLOP/s"] / (2 * PEAK_BF16_TFLOPS), 4)
+    del a8, g8, wgrad
     hin, hout = w.hidden_in - 4, w.hidden_out - 4
     au, bu = w.a[:, :hin].contiguous(), w.b[:, :hin, :hout].contiguous()
     res[f"hidden sizes {hin} x {hout} (general kernels)"] = timed(lambda: backend.gmm(au, bu, sd), reps=2,

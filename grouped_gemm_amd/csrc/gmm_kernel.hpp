@@ -608,7 +608,10 @@ struct DepthMajor {
   }
 };
 
-template <int W, int BK, int NT>
+// F8 (one-byte elements, seen two to one as W two-byte elements per depth row): 32-byte segment
+// s of depth row k sits at segment slot s ^ (k & 7), so the 8 depth rows one byte-wise
+// transposing read touches land in 8 distinct groups of 8 banks.
+template <int W, int BK, int NT, bool F8 = false>
 struct WidthMajor {
   static constexpr int CPRW = W / 8;                  // chunks per depth row
   static constexpr int SEGS = W * 2 / 64;             // 64-byte segments per depth row
@@ -621,6 +624,15 @@ struct WidthMajor {
 
   __device__ static __forceinline__ int seg_swizzle(int krow) {
     return (krow & 3) | (SEGS >= 8 ? ((krow >> 1) & 4) : 0);
+  }
+  // which 16-byte chunk of depth row krow the lane whose LDS slot is chunk p fetches
+  __device__ static __forceinline__ int chunk_for_slot(int p, int krow) {
+    if constexpr (F8) {
+      static_assert(!F8 || CPRW == 16, "8 segments of 32 bytes per depth row");
+      return (((p >> 1) ^ (krow & 7)) << 1) | (p & 1);
+    } else {
+      return (((p >> 2) ^ seg_swizzle(krow)) << 2) | (p & 3);
+    }
   }
 
   const char* base;      // depth row 0 of the group, column 0
@@ -638,7 +650,7 @@ struct WidthMajor {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int krow = krow0 + i * ROWS_PER_INSTR;
-      const int c = (((p >> 2) ^ seg_swizzle(krow)) << 2) | (p & 3);
+      const int c = chunk_for_slot(p, krow);
       const int col = col0 + c * 8;
       voff[i] = col < width ? (uint32_t)(krow * ld + col) * 2u : kOutOfRange;
     }
@@ -657,7 +669,8 @@ struct WidthMajor {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int krow = krow0 + i * ROWS_PER_INSTR;
-      const int c = (((p >> 2) ^ seg_swizzle(krow)) << 2) | (p & 3);   // 16-byte chunk of the tile row
+      static_assert(!F8, "gate | up columns are for two-byte elements");
+      const int c = chunk_for_slot(p, krow);   // 16-byte chunk of the tile row
       const int block = c >> 2;                                        // 32-column block of the tile
       const int out = col0 + (block >> 1) * 32 + (c & 3) * 8;          // output column it belongs to
       const int col = (block & 1) * out_cols + out;
@@ -736,6 +749,39 @@ struct WidthMajorFrag {
     const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
         (__attribute__((address_space(3))) bf16x4*)GG_LDS_PTR(p + 4 * PITCH));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+};
+
+// One-byte elements, width-major tile of W bytes per depth row (128 depth rows a slice).  The
+// fragment of a 32x32x64 instruction is, per lane, 32 consecutive depth values of one column
+// (depth 32 (l / 32) .. +31 of the 64-deep step, column l % 32), carried as two 16-byte halves
+// like the depth-major one: "step" 2 s + h is half h of 64-deep step s.  ds_read_b64_tr_b8 gives
+// a lane 8 consecutive depth values of its column: 16 lanes hand in the addresses of an 8 x 16
+// byte block (lane i: depth row i / 2, bytes 8 (i % 2) .. +7) and lane j of them receives column
+// j.  Two such reads make a half.
+template <int W, int NBLK, int STRIDE>
+struct WidthMajorFrag8 {
+  static constexpr int PITCH = W;
+  uint32_t off[NBLK];   // lane offset per 32-wide block, 64-deep step 0, half 0, first read
+
+  __device__ __forceinline__ void setup(int first_col) {
+    const int lane = threadIdx.x & 63;
+    const int g = lane >> 4, i = lane & 15;
+    const int krow = 32 * (g >> 1) + (i >> 1);   // (+ multiples of 8: the swizzle sees i / 2 only)
+#pragma unroll
+    for (int j = 0; j < NBLK; ++j) {
+      const int col = first_col + j * STRIDE * 32 + 16 * (g & 1) + 8 * (i & 1);
+      off[j] = (uint32_t)(krow * PITCH + ((((col >> 5) ^ (krow & 7)) << 5) | (col & 31)));
+    }
+  }
+  __device__ __forceinline__ bf16x8 read(const char* tile, int ks, int blk) const {
+    using i32x2 = __attribute__((ext_vector_type(2))) int;
+    using i32x4 = __attribute__((ext_vector_type(4))) int;
+    const char* p = tile + off[blk] + (64 * (ks / 2) + 16 * (ks % 2)) * PITCH;
+    const i32x2 lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)GG_LDS_PTR(p));
+    const i32x2 hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+        (__attribute__((address_space(3))) i32x2*)GG_LDS_PTR(p + 8 * PITCH));
+    return __builtin_bit_cast(bf16x8, i32x4{lo[0], lo[1], hi[0], hi[1]});
   }
 };
 
@@ -912,15 +958,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // as two-byte elements, two to one: same bytes per row and slice, BK_ELEMS depth values a slice.
   constexpr bool F8 = is_f8(DT);
   constexpr int ES = F8 ? 1 : 2, BK_ELEMS = BK * 2 / ES, OUT_DT = DT == kF16 ? kF16 : kBF16;
-  static_assert(!F8 || (LAYOUT == kNT && EPI == kEpiStore && !INDEXED), "fp8 streams in the NT layout, plain store");
+  static_assert(!F8 || (EPI == kEpiStore && !INDEXED), "fp8 streams with the plain store, rows in place");
   static_assert(!ACC_F32 || LAYOUT == kTN, "the fp32 accumulator is the weight gradient's");
   static_assert(!(GATE_UP || INDEXED) || LAYOUT != kTN, "row indices and gate | up are for the NN and NT layouts");
   static_assert(!GATE_UP || NB % 2 == 0, "a wave needs the gate and the up block of its columns");
   constexpr int BNS = GATE_UP ? BN / 2 : BN;   // output columns per tile, what the schedule counts in
-  using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT, INDEXED>, WidthMajor<BM, BK, NT>>;
-  using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT, false, GATE_UP>, WidthMajor<BN, BK, NT>>;
-  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK, WAVES_M, F8>, WidthMajorFrag<BM, BK, MB, WAVES_M>>;
-  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK, 1, F8>, WidthMajorFrag<BN, BK, NB, 1>>;
+  // (width-major tiles of one-byte elements: half as many two-byte elements per depth row, twice
+  // the depth rows)
+  using ALoad = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajor<BM, BK, NT, INDEXED>,
+                                   WidthMajor<BM * ES / 2, BK_ELEMS, NT, F8>>;
+  using BLoad = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajor<BN, BK, NT, false, GATE_UP>,
+                                   WidthMajor<BN * ES / 2, BK_ELEMS, NT, F8>>;
+  using AFrag = std::conditional_t<Cfg::A_DEPTH_MAJOR, DepthMajorFrag<BK, WAVES_M, F8>,
+                                   std::conditional_t<F8, WidthMajorFrag8<BM, MB, WAVES_M>, WidthMajorFrag<BM, BK, MB, WAVES_M>>>;
+  using BFrag = std::conditional_t<Cfg::B_DEPTH_MAJOR, DepthMajorFrag<BK, 1, F8>,
+                                   std::conditional_t<F8, WidthMajorFrag8<BN, NB, 1>, WidthMajorFrag<BN, BK, NB, 1>>>;
   constexpr int LOADS_PER_STAGE = ALoad::NI + BLoad::NI;   // per lane, per depth slice
   constexpr int QUARTER_LOADS = LOADS_PER_STAGE / 4;
   static_assert(KS == 4 && STAGES == 2, "the step schedule below is written for BK = 64 and two buffers");
@@ -976,7 +1028,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * ES, fti.g.k * ES / 2, fti.rows_valid,
                   depth * ES / 2);
     } else {
-      aload.setup(p.a + fti.g.a_off * 2, fti.g.m, depth, fti.m0, fti.g.m);
+      aload.setup(p.a + fti.g.a_off * ES, fti.g.m * ES / 2, depth, fti.m0 * ES / 2, fti.g.m * ES / 2);
     }
     if constexpr (GATE_UP && Cfg::B_DEPTH_MAJOR) {
       bload.setup_gate_up(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
@@ -987,7 +1039,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       bload.setup(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * ES, fti.g.k * ES / 2,
                   fti.valid && depth > 0 ? min(BN, fti.g.n - fti.n0) : 0, depth * ES / 2);
     } else {
-      bload.setup(p.b + fti.g.b_off * 2, fti.g.n, depth, fti.n0, fti.g.n);
+      bload.setup(p.b + fti.g.b_off * ES, fti.g.n * ES / 2, depth, fti.n0 * ES / 2, fti.g.n * ES / 2);
     }
   };
   // Slices past the depth (or past the last tile) are fetched with an empty descriptor:

@@ -133,7 +133,8 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  *                 Any size below 2^22 (the reference's default build runs any size through
  *                 cuBLAS, csrc/grouped_gemm.cu:373-394, its grouped kernel assumes multiples of
  *                 8, :469).  Multiples of 8 with 16-byte aligned two-byte operands run on the
- *                 streaming kernels; everything else on slower, general ones.
+ *                 streaming kernels, and so do fp8 operands whose contiguous dimensions are
+ *                 multiples of 16; everything else on slower, general ones.
  *   a_row_index   int32[tokens] on the device, or NULL: row r of the product's left operand is
  *                 row a_row_index[r] of `a` (a gather fused into the load: `a` is the tensor
  *                 before the permutation that sorts rows by group, and may have any number of

@@ -937,21 +937,28 @@ def test_float8_operands(ops, oracle, layout, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
-def test_float8_streaming_kernel(ops, oracle, dtype):
-    # the NT layout with depths that are multiples of 16 runs on the streaming kernel with the
-    # 32x32x64 fp8 matrix instruction: every count of row blocks, ragged depth and width, the
-    # DeepSeek-style shape shrunk, device- and host-resident sizes
-    cases = [([1, 31, 33, 64, 97, 128, 160, 200, 255, 256, 257, 300, 0, 513], 192, 328),
-             ([300, 0, 17, 1000], 528, 776), ([5] * 70, 272, 136), ([4000], 1024, 512), ([256] * 16, 448, 128)]
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_float8_streaming_kernel(ops, oracle, layout, dtype):
+    # hidden sizes that are multiples of 16 run on the streaming kernel with the 32x32x64 fp8 matrix
+    # instruction (width-major operands through the byte-wise transposing LDS read): every count
+    # of row blocks, ragged depth and width, the DeepSeek-style shape shrunk, device- and
+    # host-resident sizes
+    trans_a, trans_b = layout
+    cases = [([1, 31, 33, 64, 97, 128, 160, 200, 255, 256, 257, 300, 0, 513], 192, 336),
+             ([300, 0, 17, 1000], 528, 784), ([5] * 70, 272, 144), ([4000], 1024, 512), ([256] * 16, 448, 128)]
     for idx, (sizes, hin, hout) in enumerate(cases):
-        _announce("fp8 streaming", dtype, sizes, hin, hout)
+        _announce("fp8 streaming", layout, dtype, sizes, hin, hout)
         g = torch.Generator().manual_seed(idx)
         bs = torch.tensor(sizes, dtype=torch.int64)
         t = int(bs.sum())
         a = torch.randn(t, hin, generator=g).to(dtype)
-        b = torch.randn(len(sizes), hout, hin, generator=g).to(dtype)
-        out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda() if idx % 2 else bs, trans_b=True)
-        check(out, oracle.gmm_loop(a, b, bs, trans_b=True), f"case {idx}")
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(dtype)
+        else:
+            b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(dtype)
+        out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda() if idx % 2 else bs, trans_a=trans_a, trans_b=trans_b)
+        assert out.dtype == torch.bfloat16
+        check(out, oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b), f"case {idx}")
     # exact: one-hot rows against an identity-like weight give the row's value back in its place
     sizes = [1, 31, 33, 97, 160, 255, 257, 300]
     bs = torch.tensor(sizes, dtype=torch.int64)
@@ -959,9 +966,24 @@ def test_float8_streaming_kernel(ops, oracle, dtype):
     idx = torch.arange(t) % 251
     rows = torch.zeros(t, hin)
     rows[torch.arange(t), idx % hin] = (idx % 7 + 1).float()
+    if trans_a:
+        # c[e] = rows_e^T @ marks_e with marks one-hot too: c[e][i][j] counts value * 1 over the
+        # rows of group e that have their value in column i and their mark in column j
+        marks = torch.zeros(t, hout)
+        marks[torch.arange(t), (idx * 5) % hout] = 1.0
+        got = ops.backend.gmm(rows.to(dtype).cuda(), marks.to(dtype).cuda(), bs.cuda(), trans_a=True).float().cpu()
+        want = torch.zeros(len(sizes), hin, hout)
+        start = 0
+        for e, m in enumerate(sizes):
+            want[e] = rows[start:start + m].t() @ marks[start:start + m]
+            start += m
+        assert float(want.max()) <= 256.0          # sums of small integers: exact in bf16
+        assert torch.equal(got, want)
+        return
     eye = torch.zeros(len(sizes), hout, hin)
     eye[:, :hin, :] = torch.eye(hin)
-    got = ops.backend.gmm(rows.to(dtype).cuda(), eye.to(dtype).cuda(), bs.cuda(), trans_b=True).float().cpu()
+    weight = eye if trans_b else eye.transpose(1, 2).contiguous()
+    got = ops.backend.gmm(rows.to(dtype).cuda(), weight.to(dtype).cuda(), bs.cuda(), trans_b=trans_b).float().cpu()
     want = torch.zeros(t, hout)
     want[:, :hin] = rows
     assert torch.equal(got, want)
