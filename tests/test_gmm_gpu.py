@@ -989,6 +989,36 @@ def test_float8_streaming_kernel(ops, oracle, layout, dtype):
     assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("config", [2, 5])
+def test_float8_full_size(ops, oracle, config):
+    """fp8 e4m3 at the Mixtral and the DeepSeek-style shape, all three launches of forward +
+    backward: against the fp32 loop on the decoded bytes (on the GPU) and CPU float64 spot checks."""
+    from grouped_gemm_amd import workloads
+    _announce("fp8 full size", config)
+    w = workloads.make(config, device="cuda")
+    dt = torch.float8_e4m3fn
+    sizes, bs = w.batch_sizes, w.batch_sizes.cuda()
+    # (scaled up so that the values use the format's normal range, as a scaled fp8 tensor would)
+    a8, b8, g8 = (w.a.float() * 32).to(dt), (w.b.float() * 32).to(dt), (w.grad.float() * 32).to(dt)
+    with torch.no_grad():
+        out = ops.backend.gmm(a8, b8, bs, trans_b=w.trans_b)
+        check(out, oracle.gmm_loop(a8, b8, sizes, trans_b=w.trans_b), "fp8 forward")
+        fp64_rows_check(a8, b8, sizes, w.trans_b, out)
+        del out
+        ag = ops.backend.gmm(g8, b8, bs, trans_b=not w.trans_b)
+        check(ag, oracle.gmm_loop(g8, b8, sizes, trans_b=not w.trans_b), "fp8 agrad")
+        fp64_rows_check(g8, b8, sizes, not w.trans_b, ag, seed=1)
+        del ag
+        lhs, rhs = (g8, a8) if w.trans_b else (a8, g8)
+        bg = ops.backend.gmm(lhs, rhs, bs, trans_a=True)
+        starts = torch.cumsum(sizes, 0) - sizes
+        for e in range(0, len(sizes), max(1, len(sizes) // 8)):
+            s0, m = int(starts[e]), int(sizes[e])
+            check(bg[e], lhs[s0:s0 + m].float().t() @ rhs[s0:s0 + m].float(), f"fp8 bgrad expert {e}")
+        fp64_weight_gradient_check(lhs, rhs, sizes, bg)
+        assert torch.equal(bg, ops.backend.gmm(lhs, rhs, sizes, trans_a=True))
+
+
 # ------------------------------------------------------------- fused gather / scatter
 
 def _routing(tokens, experts, top_k, seed):
