@@ -207,7 +207,8 @@ def other_paths(steps=5, warmup=2):
     """The paths past the reference's surface, timed shortly on the forward GEMM of the default
     workload (8 experts, 32768 rows, 4096 x 14336): fused row gather and scatter, the SwiGLU
     epilogue (the same b read as gate | up, so half the output width), float16, fp8 (e4m3, b as
-    stored and b stored transposed, and the weight gradient), and hidden sizes that are not multiples of 8 (the general kernels)."""
+    stored and b stored transposed, and the weight gradient), and hidden sizes that are not
+    multiples of 8 (through zero-padded copies, and on the general kernels)."""
     import torch
     from grouped_gemm import backend
     from grouped_gemm_amd import workloads
@@ -253,8 +254,12 @@ def other_paths(steps=5, warmup=2):
     del a8, g8, wgrad
     hin, hout = w.hidden_in - 4, w.hidden_out - 4
     au, bu = w.a[:, :hin].contiguous(), w.b[:, :hin, :hout].contiguous()
+    res[f"hidden sizes {hin} x {hout} (zero-padded copies, streaming kernel)"] = timed(
+        lambda: backend.gmm(au, bu, sd), reps=2, f=2 * t * hin * hout)
+    backend.PAD_ODD_SIZES = False
     res[f"hidden sizes {hin} x {hout} (general kernels)"] = timed(lambda: backend.gmm(au, bu, sd), reps=2,
                                                                  f=2 * t * hin * hout)
+    backend.PAD_ODD_SIZES = True
     return res
 
 

@@ -832,7 +832,14 @@ def test_float16_autograd_and_mixed_dtypes(ops, oracle, trans_b):
     assert float((c.double().cpu() - want_c).abs().max()) <= 1e-4 * float(want_c.abs().max())
 
 
-# ------------------------------------- any hidden size, any alignment (the general kernels)
+# ---- any hidden size, any alignment (the general kernels, and gmm's zero-padded copies instead)
+
+@pytest.fixture(params=[False, True], ids=["general-kernels", "padded-copies"])
+def odd_size_path(request, ops, monkeypatch):
+    """Both ways backend.gmm serves operands the streaming kernels do not take."""
+    monkeypatch.setattr(ops.backend, "PAD_ODD_SIZES", request.param)
+    return request.param
+
 
 def _odd_cases(n, seed):
     g = torch.Generator().manual_seed(seed)
@@ -850,7 +857,7 @@ def _odd_cases(n, seed):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
-def test_hidden_sizes_that_are_not_multiples_of_8(ops, oracle, layout, dtype):
+def test_hidden_sizes_that_are_not_multiples_of_8(ops, oracle, layout, dtype, odd_size_path):
     # the reference's default build takes any hidden size (csrc/grouped_gemm.cu:373-394); sizes
     # that are multiples of 4, of 2, and odd ones, each through its own vector width
     trans_a, trans_b = layout
@@ -871,7 +878,7 @@ def test_hidden_sizes_that_are_not_multiples_of_8(ops, oracle, layout, dtype):
 
 
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
-def test_operands_off_the_16_byte_boundary(ops, oracle, layout):
+def test_operands_off_the_16_byte_boundary(ops, oracle, layout, odd_size_path):
     # views that start one, two or four elements into a buffer: same results as the aligned call
     trans_a, trans_b = layout
     g = torch.Generator().manual_seed(61)
@@ -896,6 +903,22 @@ def test_operands_off_the_16_byte_boundary(ops, oracle, layout):
         check(c, want, f"shifted by {by_a}, {by_b}, {by_c} elements")
 
 
+def test_padded_copies_leave_tail_rows_alone(ops, oracle):
+    # sum(batch_sizes) < rows of a: the rows of c past the sum keep their contents on this path too
+    g = torch.Generator().manual_seed(64)
+    sizes = torch.tensor([40, 0, 25])
+    a = torch.randn(100, 33, generator=g).to(torch.bfloat16)
+    b = torch.randn(3, 33, 50, generator=g).to(torch.bfloat16)
+    c = torch.full((100, 50), 7.0, dtype=torch.bfloat16, device="cuda")
+    assert ops.backend.PAD_ODD_SIZES
+    ops.backend.gmm(a.cuda(), b.cuda(), sizes.cuda(), c=c)
+    check(c[:65], oracle.gmm_loop(a, b, sizes)[:65], "rows in use")
+    assert bool((c[65:] == 7.0).all())
+    # malformed calls raise what the plain path raises
+    with pytest.raises(RuntimeError):
+        ops.backend.gmm(a.cuda(), b.cuda()[:, :32], sizes.cuda())
+
+
 def test_accumulated_weight_gradient_any_size(ops, oracle):
     g = torch.Generator().manual_seed(63)
     sizes = torch.tensor([300, 0, 17, 129])
@@ -915,7 +938,7 @@ def test_accumulated_weight_gradient_any_size(ops, oracle):
 
 @pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
-def test_float8_operands(ops, oracle, layout, dtype):
+def test_float8_operands(ops, oracle, layout, dtype, odd_size_path):
     # fp8 in a and b (OCP formats), fp32 accumulation of the exact products, one bf16 rounding on
     # store; the oracle is the per-expert loop on the fp32 decode of the same bytes
     trans_a, trans_b = layout
