@@ -968,7 +968,10 @@ def test_float8_streaming_kernel(ops, oracle, layout, dtype):
     # host-resident sizes
     trans_a, trans_b = layout
     cases = [([1, 31, 33, 64, 97, 128, 160, 200, 255, 256, 257, 300, 0, 513], 192, 336),
-             ([300, 0, 17, 1000], 528, 784), ([5] * 70, 272, 144), ([4000], 1024, 512), ([256] * 16, 448, 128)]
+             ([300, 0, 17, 1000], 528, 784), ([5] * 70, 272, 144), ([4000], 1024, 512), ([256] * 16, 448, 128),
+             # few tiles and a deep product: the last round is cut along the depth (100 slices of
+             # 128 in the NN and NT layouts, 102 in the weight-gradient layout)
+             ([300, 200], 12800, 256), ([13000], 256, 256)]
     for idx, (sizes, hin, hout) in enumerate(cases):
         _announce("fp8 streaming", layout, dtype, sizes, hin, hout)
         g = torch.Generator().manual_seed(idx)
