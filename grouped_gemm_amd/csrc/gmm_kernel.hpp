@@ -958,7 +958,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // as two-byte elements, two to one: same bytes per row and slice, BK_ELEMS depth values a slice.
   constexpr bool F8 = is_f8(DT);
   constexpr int ES = F8 ? 1 : 2, BK_ELEMS = BK * 2 / ES, OUT_DT = DT == kF16 ? kF16 : kBF16;
-  static_assert(!F8 || (EPI == kEpiStore && !INDEXED), "fp8 streams with the plain store, rows in place");
+  static_assert(!F8 || (!GATE_UP && !INDEXED), "fp8 streams with rows in place and no gate | up columns");
   static_assert(!ACC_F32 || LAYOUT == kTN, "the fp32 accumulator is the weight gradient's");
   static_assert(!(GATE_UP || INDEXED) || LAYOUT != kTN, "row indices and gate | up are for the NN and NT layouts");
   static_assert(!GATE_UP || NB % 2 == 0, "a wave needs the gate and the up block of its columns");

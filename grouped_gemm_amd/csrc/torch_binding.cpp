@@ -242,7 +242,7 @@ void GroupedGemmSwiGLU(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch:
 void AccumulateWeightGradient(torch::Tensor a, torch::Tensor b, torch::Tensor c, torch::Tensor batch_sizes) {
   TORCH_CHECK(c.scalar_type() == torch::kFloat32, "grouped_gemm: the accumulated gradient must be float32");
   // every other check is the one of the bf16 weight-gradient call
-  torch::Tensor shape_of_c = torch::empty(c.sizes(), torch::dtype(a.scalar_type()).device(torch::kMeta));
+  torch::Tensor shape_of_c = torch::empty(c.sizes(), torch::dtype(OutputType(a.scalar_type())).device(torch::kMeta));
   Validate(a, b, shape_of_c, batch_sizes, /*trans_a=*/true, /*trans_b=*/false, /*on_device=*/false);
   TORCH_CHECK(a.is_cuda() && b.is_cuda() && c.is_cuda(), "grouped_gemm: a, b and c must be GPU tensors");
   TORCH_CHECK(b.device() == a.device() && c.device() == a.device(),

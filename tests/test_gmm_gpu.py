@@ -1284,6 +1284,27 @@ def test_accumulated_weight_gradient(ops, oracle, sizes, hin, hout, on_device):
     assert (second - 2 * first).abs().max().item() <= 4 * tol
 
 
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+def test_accumulated_weight_gradient_float8(ops, oracle, dtype):
+    # fp8 operands added to an fp32 weight gradient: shallow groups (read-add-write), deep ones
+    # (atomic additions), sizes the streaming kernels take and sizes they do not
+    g = torch.Generator().manual_seed(66)
+    for sizes, hin, hout in [([300, 0, 17, 129], 272, 144), ([3000, 2500], 256, 512), ([70, 5], 100, 24)]:
+        _announce("accumulate fp8", dtype, sizes, hin, hout)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        b = torch.randn(t, hout, generator=g).to(dtype)
+        c0 = torch.randn(len(sizes), hin, hout, generator=g)
+        c = c0.clone().cuda()
+        ops.backend.accumulate_weight_gradient(a.cuda(), b.cuda(), bs.cuda(), c)
+        want = oracle.accumulate_weight_gradient_loop(a, b, bs, c0)
+        assert float((c.double().cpu() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+        for e, m in enumerate(sizes):
+            if m == 0:
+                assert torch.equal(c[e].cpu(), c0[e])
+
+
 def test_accumulated_weight_gradient_full_size_and_errors(ops, oracle):
     from grouped_gemm_amd import workloads
     w = workloads.make(4, device="cuda")                # 8 x 4096 rows, 4096 x 14336
