@@ -1053,7 +1053,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // Load J of the cursor's slice (A's loads first, then B's) into buffer `buf`.
   auto fetch_load = [&](auto j_tag, int buf) {
     constexpr int J = decltype(j_tag)::value;
-    const char* st = smem + buf * Cfg::STAGE_BYTES;
+    const char* st = smem + uniform(buf) * Cfg::STAGE_BYTES;
     if constexpr (kDiagnosticNoLoads) {
     } else if constexpr (J < ALoad::NI) {
       aload.template load<J>(a_slice, st, wave);
@@ -1062,8 +1062,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     }
   };
   auto fetch_advance = [&]() {
-    if (++fetch_kt == fti.nk && fti.valid) {
-      fetch_t += G;
+    // (said to be the same in every lane once more: where the compiler loses track of that, the
+    // slice descriptors below are computed lane by lane and the branch becomes a masked one)
+    fetch_kt = uniform(fetch_kt + 1);
+    if (fetch_kt == uniform(fti.nk) && uniform((int)fti.valid) != 0) {
+      fetch_t = uniform(fetch_t + G);
       fetch_kt = 0;
       fetch_setup();
     }
@@ -1187,7 +1190,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     };
 
     for (int kt = 0; kt < ti.nk; ++kt) {
-      const int y = x ^ 1;
+      const int y = uniform(x ^ 1);   // (the same in every lane: keeps the LDS addresses scalar)
       step(I0{}, I2{}, ml_tag, I2{}, IQ3{}, IQ{}, x, y);
       fetch_advance();
       // every wave has all fragments of this slice in registers
@@ -1200,7 +1203,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       wait_vmcnt<2 * QUARTER_LOADS>();
       block_barrier();
       step(I3{}, I2{}, IMB{}, I0{}, IQ2{}, IQ{}, y, x);
-      x = y;
+      x = uniform(y);
     }
 
     // A depth piece of a tile of the last round: park the partial tile in the workspace and
@@ -1421,7 +1424,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
         tile_body(std::integral_constant<int, 1>{});
       }
     }
-    tile_t += G;
+    tile_t = uniform(tile_t + G);
     if (tile_t >= total_tiles) break;
     ti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, tile_t, plan, tile_cur);
   }
