@@ -795,6 +795,8 @@ __device__ __forceinline__ void static_for(F&& f) {
   }(std::make_integer_sequence<int, N>{});
 }
 
+constexpr int kTileInfoDwords = 24;   // a tile's description on its way through LDS (pack_tile)
+
 template <int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N>
 struct GmmConfig {
   static constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -811,9 +813,13 @@ struct GmmConfig {
   static constexpr int EPILOGUE_WAVE_BYTES = 32 * EPILOGUE_PITCH;
   static constexpr bool STAGED_EPILOGUE =
       NB % 2 == 0 && EPILOGUE_OFFSET + WAVES_M * WAVES_N * EPILOGUE_WAVE_BYTES <= 160 * 1024;
-  static constexpr int LDS_BYTES =
-      STAGED_EPILOGUE ? EPILOGUE_OFFSET + WAVES_M * WAVES_N * EPILOGUE_WAVE_BYTES
-                      : SCHED_OFFSET + (int)sizeof(Sched);
+  // last: per wave, the descriptions of the tiles between the fetch and the compute cursor
+  static constexpr int TILE_RING_SLOTS = 4;
+  static constexpr int TILE_RING_OFFSET =
+      ((STAGED_EPILOGUE ? EPILOGUE_OFFSET + WAVES_M * WAVES_N * EPILOGUE_WAVE_BYTES
+                        : SCHED_OFFSET + (int)sizeof(Sched)) + 15) / 16 * 16;
+  static constexpr int LDS_BYTES = TILE_RING_OFFSET + WAVES_M * WAVES_N * TILE_RING_SLOTS * kTileInfoDwords * 4;
+  static_assert(LDS_BYTES <= 160 * 1024, "a compute unit has 160 KiB of LDS");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32 MFMA blocks");
   static_assert(BK % 16 == 0 && STAGES >= 2, "");
 };
@@ -839,6 +845,28 @@ struct TileCursor {
   int e = 0;
   int cls = 0;
 };
+
+// A tile's description as 24 dwords, for the trip through LDS from the fetch cursor, which works
+// it out, to the compute cursor, which needs the same one or two tiles later.
+__device__ __forceinline__ void pack_tile(const TileInfo& t, int32_t* w) {
+  w[0] = (int32_t)t.g.a_off, w[1] = (int32_t)(t.g.a_off >> 32);
+  w[2] = (int32_t)t.g.b_off, w[3] = (int32_t)(t.g.b_off >> 32);
+  w[4] = (int32_t)t.g.c_off, w[5] = (int32_t)(t.g.c_off >> 32);
+  w[6] = t.g.m, w[7] = t.g.n, w[8] = t.g.k, w[9] = t.g.row0;
+  w[10] = t.m0, w[11] = t.n0, w[12] = t.rows_valid, w[13] = t.blocks, w[14] = t.depth, w[15] = t.k0;
+  w[16] = t.nk, w[17] = t.pieces, w[18] = t.piece, w[19] = t.rank, w[20] = t.valid ? 1 : 0;
+  w[21] = w[22] = w[23] = 0;
+}
+__device__ __forceinline__ TileInfo unpack_tile(const int32_t* w) {
+  auto u = [&](int i) { return uniform(w[i]); };
+  auto u64 = [&](int i) { return (int64_t)(((uint64_t)(uint32_t)u(i + 1) << 32) | (uint32_t)u(i)); };
+  TileInfo t;
+  t.g.a_off = u64(0), t.g.b_off = u64(2), t.g.c_off = u64(4);
+  t.g.m = u(6), t.g.n = u(7), t.g.k = u(8), t.g.row0 = u(9);
+  t.m0 = u(10), t.n0 = u(11), t.rows_valid = u(12), t.blocks = u(13), t.depth = u(14), t.k0 = u(15);
+  t.nk = u(16), t.pieces = u(17), t.piece = u(18), t.rank = u(19), t.valid = u(20) != 0;
+  return t;
+}
 
 // Tile index -> group and position.  Indices past plan.main_tiles name pieces of the last
 // round's tiles: piece (t - main) % pieces of tile main + (t - main) / pieces.
@@ -1017,8 +1045,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   int fetch_t = vid, fetch_kt = 0;
   TileCursor fetch_cur;
   TileInfo fti;
+  // The compute cursor does not look its tiles up again: the fetch cursor, which is one or two
+  // tiles ahead, leaves each description in a ring in LDS (one ring per wave, written by its first
+  // lane and read back by the same wave: no barrier involved).
+  int32_t* tile_ring = reinterpret_cast<int32_t*>(smem + Cfg::TILE_RING_OFFSET) +
+                       wave * (Cfg::TILE_RING_SLOTS * kTileInfoDwords);
+  int fetch_n = 0;   // tiles the fetch cursor has set up
   auto fetch_setup = [&]() {
     fti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, fetch_t, plan, fetch_cur);
+    {
+      int32_t words[kTileInfoDwords];
+      pack_tile(fti, words);
+      int32_t* slot = tile_ring + (fetch_n % Cfg::TILE_RING_SLOTS) * kTileInfoDwords;
+      if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < kTileInfoDwords; i += 4)
+          *reinterpret_cast<u32x4*>(slot + i) = u32x4{(uint32_t)words[i], (uint32_t)words[i + 1],
+                                                      (uint32_t)words[i + 2], (uint32_t)words[i + 3]};
+      }
+      fetch_n = uniform(fetch_n + 1);
+    }
     const int depth = fti.depth;
     if constexpr (INDEXED) {
       const int first = fti.g.row0 + fti.m0;
@@ -1105,8 +1151,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   static_for<3 * QUARTER_LOADS>([&](auto j) { fetch_load(j, 1); });
 
   int tile_t = vid;
-  TileCursor tile_cur;
-  TileInfo ti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, tile_t, plan, tile_cur);
+  int tile_n = 0;   // tiles this workgroup has finished
+  auto next_tile = [&]() {
+    int32_t words[kTileInfoDwords];
+    const int32_t* slot = tile_ring + (tile_n % Cfg::TILE_RING_SLOTS) * kTileInfoDwords;
+#pragma unroll
+    for (int i = 0; i < kTileInfoDwords; i += 4) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(slot + i);
+      words[i] = (int32_t)v[0], words[i + 1] = (int32_t)v[1], words[i + 2] = (int32_t)v[2], words[i + 3] = (int32_t)v[3];
+    }
+    return unpack_tile(words);
+  };
+  TileInfo ti = next_tile();
   wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
   static_for<2 * UNITS>([&](auto u) {
@@ -1426,7 +1482,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     }
     tile_t = uniform(tile_t + G);
     if (tile_t >= total_tiles) break;
-    ti = find_tile<LAYOUT, BM, BNS, BK_ELEMS>(sched, p, tile_t, plan, tile_cur);
+    tile_n = uniform(tile_n + 1);
+    ti = next_tile();
   }
   wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
 
