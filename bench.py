@@ -203,7 +203,7 @@ def summarize(w, names, layout, ms_per_step, samples, accumulate=False):
     return value, roofline, slowest, kernel_ms
 
 
-def other_paths(steps=5, warmup=2):
+def other_paths(steps=7, warmup=4):
     """The paths past the reference's surface, timed shortly on the forward GEMM of the default
     workload (8 experts, 32768 rows, 4096 x 14336): fused row gather and scatter, the SwiGLU
     epilogue (the same b read as gate | up, so half the output width), float16, fp8 (e4m3, b as
