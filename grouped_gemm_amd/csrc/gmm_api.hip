@@ -202,13 +202,13 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   // that are multiples of 8, operands on 16-byte boundaries, rows in place.  Everything else goes
   // to the kernels of gmm_generic.hpp, VEC elements at a time.
   const bool indexed = g.a_row_index != nullptr || g.b_row_index != nullptr || g.c_row_index != nullptr;
-  const int64_t a_bytes = (g.a_num_rows > 0 ? g.a_num_rows : tokens) * hidden_in * 2;
+  const int64_t a_bytes = (g.a_num_rows > 0 ? g.a_num_rows : tokens) * hidden_in * elem_bytes;
   const int64_t c_bytes = (g.c_num_rows > 0 ? g.c_num_rows : tokens) * hidden_out * 2;
   // with row indices the streaming kernels address a and c through 32-bit byte offsets
   const bool indexed_fits = !trans_a && a_bytes < (int64_t)gg::kOutOfRangeIndexed && c_bytes < (int64_t)gg::kOutOfRangeIndexed;
   // (fp8 streams in 16-byte chunks like the rest: 16 elements, along whichever dimension is
   // contiguous in each operand)
-  const bool f8_streams = elem_bytes == 1 && !indexed && !swiglu &&
+  const bool f8_streams = elem_bytes == 1 && !swiglu &&
                           (trans_a ? hidden_in % 16 == 0 && hidden_out % 16 == 0
                                    : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
   const bool generic = (elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||

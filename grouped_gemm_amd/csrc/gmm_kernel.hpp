@@ -986,7 +986,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // as two-byte elements, two to one: same bytes per row and slice, BK_ELEMS depth values a slice.
   constexpr bool F8 = is_f8(DT);
   constexpr int ES = F8 ? 1 : 2, BK_ELEMS = BK * 2 / ES, OUT_DT = DT == kF16 ? kF16 : kBF16;
-  static_assert(!F8 || (!GATE_UP && !INDEXED), "fp8 streams with rows in place and no gate | up columns");
+  static_assert(!F8 || !GATE_UP, "fp8 streams without gate | up columns");
   static_assert(!ACC_F32 || LAYOUT == kTN, "the fp32 accumulator is the weight gradient's");
   static_assert(!(GATE_UP || INDEXED) || LAYOUT != kTN, "row indices and gate | up are for the NN and NT layouts");
   static_assert(!GATE_UP || NB % 2 == 0, "a wave needs the gate and the up block of its columns");
@@ -1068,8 +1068,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     const int depth = fti.depth;
     if constexpr (INDEXED) {
       const int first = fti.g.row0 + fti.m0;
-      aload.setup_gather(p.a, p.a_bytes, p.a_rows != nullptr ? p.a_rows + first : nullptr, first, fti.g.k,
-                         depth > 0 ? fti.rows_valid : 0, depth);
+      aload.setup_gather(p.a, p.a_bytes, p.a_rows != nullptr ? p.a_rows + first : nullptr, first,
+                         fti.g.k * ES / 2, depth > 0 ? fti.rows_valid : 0, depth * ES / 2);
     } else if constexpr (Cfg::A_DEPTH_MAJOR) {
       aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * ES, fti.g.k * ES / 2, fti.rows_valid,
                   depth * ES / 2);

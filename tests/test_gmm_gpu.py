@@ -1087,6 +1087,31 @@ def test_gather_and_scatter_against_indexed_oracle(ops, oracle, trans_b, hidden)
     check(c2, want_c[:800], "gathered and scattered")
 
 
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_gather_and_scatter_float8(ops, oracle, trans_b, dtype):
+    # fp8 operands with the permutation fused in, on the streaming kernels (hidden sizes multiples of
+    # 16) and on the general ones; row counts that leave ragged tiles
+    for hin, hout, tokens, experts in [(144, 272, 400, 6), (100, 24, 300, 5), (256, 512, 3000, 3)]:
+        row_index, sizes, order = _routing(tokens, experts, 2, seed=85)
+        g = torch.Generator().manual_seed(86)
+        x = torch.randn(tokens, hin, generator=g).to(dtype)
+        w = torch.randn(experts, *((hout, hin) if trans_b else (hin, hout)), generator=g).to(dtype)
+        _announce("gather fp8", dtype, trans_b, hin, hout, tokens)
+        want = oracle.gmm_loop(x[row_index.long()], w, sizes, trans_b=trans_b)
+        got = ops.backend.gmm_indexed(x.cuda(), w.cuda(), sizes.cuda(), trans_b=trans_b, a_rows=row_index.cuda())
+        assert got.dtype == torch.bfloat16
+        check(got, want, "gathered rows")
+        rows = 2 * tokens
+        c = torch.full((rows + 3, hout), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.backend.gmm_indexed(x.cuda(), w.cuda(), sizes.cuda(), trans_b=trans_b, c=c, a_rows=row_index.cuda(),
+                                c_rows=order.cuda())
+        want_c = torch.full((rows + 3, hout), 7.0)
+        want_c[order.long()] = want
+        check(c, want_c, "gathered and scattered")
+        assert (c[rows:] == 7.0).all()
+
+
 @pytest.mark.parametrize("hidden", [(136, 264), (33, 20)])
 def test_weight_gradient_with_gathered_rows(ops, oracle, hidden):
     hin, hout = hidden
