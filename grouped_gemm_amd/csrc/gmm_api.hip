@@ -208,7 +208,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   const bool indexed_fits = !trans_a && a_bytes < (int64_t)gg::kOutOfRangeIndexed && c_bytes < (int64_t)gg::kOutOfRangeIndexed;
   // (fp8 streams in 16-byte chunks like the rest: 16 elements, along whichever dimension is
   // contiguous in each operand)
-  const bool f8_streams = elem_bytes == 1 && !swiglu &&
+  const bool f8_streams = elem_bytes == 1 && (!swiglu || (trans_b && !indexed)) &&
                           (trans_a ? hidden_in % 16 == 0 && hidden_out % 16 == 0
                                    : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
   const bool generic = (elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||

@@ -986,7 +986,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // as two-byte elements, two to one: same bytes per row and slice, BK_ELEMS depth values a slice.
   constexpr bool F8 = is_f8(DT);
   constexpr int ES = F8 ? 1 : 2, BK_ELEMS = BK * 2 / ES, OUT_DT = DT == kF16 ? kF16 : kBF16;
-  static_assert(!F8 || !GATE_UP, "fp8 streams without gate | up columns");
+  static_assert(!F8 || !GATE_UP || LAYOUT == kNT, "fp8 with gate | up rows streams in the NT layout only");
   static_assert(!ACC_F32 || LAYOUT == kTN, "the fp32 accumulator is the weight gradient's");
   static_assert(!(GATE_UP || INDEXED) || LAYOUT != kTN, "row indices and gate | up are for the NN and NT layouts");
   static_assert(!GATE_UP || NB % 2 == 0, "a wave needs the gate and the up block of its columns");
@@ -1077,8 +1077,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       aload.setup(p.a + fti.g.a_off * ES, fti.g.m * ES / 2, depth, fti.m0 * ES / 2, fti.g.m * ES / 2);
     }
     if constexpr (GATE_UP && Cfg::B_DEPTH_MAJOR) {
-      bload.setup_gate_up(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * 2, fti.g.k,
-                          fti.valid && depth > 0 ? 2 * fti.g.n - fti.n0 : 0, depth, fti.g.n);
+      bload.setup_gate_up(p.b + (fti.g.b_off + (int64_t)fti.n0 * fti.g.k) * ES, fti.g.k * ES / 2,
+                          fti.valid && depth > 0 ? 2 * fti.g.n - fti.n0 : 0, depth * ES / 2, fti.g.n);
     } else if constexpr (GATE_UP) {
       bload.setup_gate_up(p.b + fti.g.b_off * 2, 2 * fti.g.n, depth, fti.n0, fti.g.n);
     } else if constexpr (Cfg::B_DEPTH_MAJOR) {

@@ -1196,6 +1196,24 @@ def test_swiglu_epilogue(ops, oracle, trans_b, dtype):
         check(out, oracle.swiglu_loop(a, b, bs, trans_b=trans_b), f"case {idx}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float8_e4m3fn, torch.float8_e5m2])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_swiglu_epilogue_float8(ops, oracle, trans_b, dtype):
+    # fp8 operands: b stored transposed runs on the streaming kernel (depth a multiple of 16), the
+    # other layout and other sizes on the general ones; the output is bfloat16
+    for idx, (sizes, hin, hout) in enumerate([([300, 0, 17, 195], 256, 384), ([1, 255, 257, 64], 144, 200),
+                                              ([1000], 528, 776), ([130, 7], 100, 12)]):
+        _announce("swiglu fp8", trans_b, dtype, sizes, hin, hout)
+        g = torch.Generator().manual_seed(idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        b = (torch.randn(len(sizes), *((2 * hout, hin) if trans_b else (hin, 2 * hout)), generator=g) * hin ** -0.5 * 4).to(dtype)
+        out = ops.backend.gmm_swiglu(a.cuda(), b.cuda(), bs.cuda() if idx % 2 else bs, trans_b=trans_b)
+        assert out.shape == (t, hout) and out.dtype == torch.bfloat16
+        check(out, oracle.swiglu_loop(a, b, bs, trans_b=trans_b), f"case {idx}")
+
+
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_swiglu_with_gathered_and_scattered_rows(ops, oracle, trans_b):
     hin, hout = 136, 264
