@@ -917,6 +917,8 @@ def test_padded_copies_leave_tail_rows_alone(ops, oracle):
     # malformed calls raise what the plain path raises
     with pytest.raises(RuntimeError):
         ops.backend.gmm(a.cuda(), b.cuda()[:, :32], sizes.cuda())
+    with pytest.raises(RuntimeError):
+        ops.backend.gmm(a.cuda().t().contiguous().t(), b.cuda(), sizes.cuda())   # a not contiguous
 
 
 def test_accumulated_weight_gradient_any_size(ops, oracle):
