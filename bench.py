@@ -49,6 +49,24 @@ MEASURED_TRAFFIC = {
 }
 
 
+def mfma_rate(zero_operands, launches):
+    """TFLOP/s of the bf16 matrix instruction alone (bench_mfma_probe.hip, built next to this file
+    by grouped_gemm_amd/build.py: a helper of the benchmark, not of the library)."""
+    import ctypes
+    path = os.path.join(ROOT, "libbench_mfma_probe.so")
+    if not os.path.exists(path):
+        from grouped_gemm_amd import build as _build
+        _build.build_bench_probe()
+    lib = ctypes.CDLL(path)
+    lib.bench_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+    lib.bench_mfma_rate.restype = ctypes.c_int
+    tflops = ctypes.c_float(0.0)
+    rc = lib.bench_mfma_rate(1 if zero_operands else 0, launches, ctypes.byref(tflops))
+    if rc != 0:
+        raise RuntimeError(f"bench_mfma_rate failed with hipError_t {rc}")
+    return tflops.value
+
+
 def cpu_baseline(w, budget_s=12.0):
     """Oracle loop on the host cores: forward, input gradient and weight gradient of the
     same workload through torch's CPU bf16 matmul.  A calibration run on a slice of expert 0
@@ -344,11 +362,9 @@ def main():
     # What the chip sustains on the matrix instruction alone (operands in registers, no memory
     # traffic), right after the timed region: on operands with the bit statistics of this data the
     # power limit lowers the clock, on zeros it does not.  The first figure is the ceiling of any
-    # bf16 GEMM on this device and data.
-    from grouped_gemm import backend as _backend
-    dev = torch.device("cuda", 0)
-    pipe_random = _backend.backend.mfma_rate(dev, False, 10)
-    pipe_zeros = _backend.backend.mfma_rate(dev, True, 10)
+    # bf16 GEMM on this device and data.  (A helper of this file, not of the library.)
+    pipe_random = mfma_rate(False, 10)
+    pipe_zeros = mfma_rate(True, 10)
     out["matrix_pipe_alone"] = {
         "what": "v_mfma_f32_32x32x16_bf16 on register operands, 256 workgroups of 4 waves, 10 launches of about 2.5 ms",
         "random_operands_TFLOP/s": round(pipe_random, 1),

@@ -4,14 +4,17 @@
 // its clock to stay inside its power limit; on all-zero operands it does not.  The first figure
 // is therefore the ceiling of any bf16 GEMM on this device and data, whatever its memory system
 // does; the benchmark prints both next to the GEMM's own rate.
+//
+// A helper of bench.py only (built as libbench_mfma_probe.so next to it, loaded through ctypes):
+// no part of libgrouped_gemm_hip.so or of its header.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
 
-#include "gmm_kernel.hpp"
-
-namespace gg {
 namespace {
+
+using bf16x8 = __attribute__((ext_vector_type(8))) __bf16;
+using f32x16 = __attribute__((ext_vector_type(16))) float;
 
 constexpr int kProbeWaves = 4, kProbeBlocks = 4;   // 4 x 4 blocks of 32 x 32 per wave: 256 accumulator registers
 
@@ -51,7 +54,7 @@ __global__ __launch_bounds__(kProbeWaves * 64) void mfma_probe_kernel(int iterat
 #pragma unroll
     for (int j = 0; j < kProbeBlocks; ++j)
 #pragma unroll
-      for (int i = 0; i < kProbeBlocks; ++i) acc[i][j] = mfma_32x32x16<kBF16>(b[j], a[i], acc[i][j]);
+      for (int i = 0; i < kProbeBlocks; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[j], a[i], acc[i][j], 0, 0, 0);
     // new operand values every step, as a depth loop would bring them (the elements of two
     // fragments rotate: register moves only)
     a[0] = __builtin_shufflevector(a[0], a[0], 1, 2, 3, 4, 5, 6, 7, 0);
@@ -65,8 +68,6 @@ __global__ __launch_bounds__(kProbeWaves * 64) void mfma_probe_kernel(int iterat
   if (s == 12345.678f) sink[0] = s;   // never true for these operands; keeps the loop alive
 #endif
 }
-
-}  // namespace
 
 // Launches the probe `launches` + 1 times on `stream` (the first untimed) with one workgroup per
 // compute unit and returns the rate of the timed ones in TFLOP/s through `tflops`.
@@ -98,4 +99,22 @@ hipError_t run_mfma_probe(int cus, int zeros, int launches, float* sink, hipStre
   return hipSuccess;
 }
 
-}  // namespace gg
+}  // namespace
+
+// TFLOP/s of `launches` probe launches of about 2 ms each on the current device's null stream
+// (waits for them); zero_operands != 0: all-zero operands.  Returns a hipError_t as int.
+extern "C" int bench_mfma_rate(int zero_operands, int launches, float* tflops) {
+  if (tflops == nullptr || launches < 1 || launches > 1000) return (int)hipErrorInvalidValue;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return (int)err;
+  hipDeviceProp_t prop;
+  err = hipGetDeviceProperties(&prop, dev);
+  if (err != hipSuccess) return (int)err;
+  float* sink = nullptr;
+  err = hipMalloc(&sink, 256);
+  if (err != hipSuccess) return (int)err;
+  err = run_mfma_probe(prop.multiProcessorCount, zero_operands != 0, launches, sink, nullptr, tflops);
+  (void)hipFree(sink);
+  return (int)err;
+}

@@ -3,16 +3,14 @@
   libgrouped_gemm_hip.so            HIP kernels + C ABI (hipcc, gfx950 only)
   grouped_gemm_backend.<abi>.so     PyTorch-ROCm binding (g++, links the first)
 
-Usage: python grouped_gemm_amd/build.py [--force] [--diagnostic no_loads|no_mfma]
+Usage: python grouped_gemm_amd/build.py [--force]
 hipcc cross-compiles gfx950 without a GPU, so this runs anywhere the ROCm toolchain
 and PyTorch-ROCm are installed.  The kernel variants (csrc/gmm_variants.def) are compiled as
 separate translation units, several at a time; objects are kept under grouped_gemm_amd/build/.
 
---diagnostic NAME builds a second copy of the kernel library with GG_DIAGNOSTIC_<NAME> defined
-(csrc/gmm_kernel.hpp: the kernels without their operand loads, or without their matrix
-instructions; wrong results, for timing only) into grouped_gemm_amd/diagnostic/NAME/.  Nothing
-loads it unless that directory is put first on LD_LIBRARY_PATH, e.g.
-LD_LIBRARY_PATH=grouped_gemm_amd/diagnostic/no_mfma python bench.py --config 5 --no-cpu-baseline
+build_bench_probe() builds bench.py's own helper (bench_mfma_probe.hip at the repository root,
+a matrix-instruction rate probe) into libbench_mfma_probe.so next to it; it is no part of the
+library.
 """
 import os
 import re
@@ -64,21 +62,14 @@ def variant_indices():
     return [int(m) for m in re.findall(r"^GG_VARIANT\((\d+),", text, flags=re.M)]
 
 
-def build_hip(force=False, jobs=None, diagnostic=None):
+def build_hip(force=False, jobs=None):
     headers = [os.path.join(CSRC, f) for f in ("gmm_kernel.hpp", "gmm_generic.hpp", "gmm_variants.hpp",
                                                "gmm_variants.def")]
     headers.append(os.path.join(ROOT, "include", "grouped_gemm_hip.h"))
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     obj_dir, hip_lib, extra = OBJ_DIR, HIP_LIB, []
-    if diagnostic:
-        if diagnostic not in ("no_loads", "no_mfma"):
-            raise ValueError("--diagnostic takes no_loads or no_mfma")
-        obj_dir = os.path.join(HERE, "diagnostic", diagnostic)
-        hip_lib = os.path.join(obj_dir, os.path.basename(HIP_LIB))
-        extra = ["-DGG_DIAGNOSTIC_" + diagnostic.upper()]
     os.makedirs(obj_dir, exist_ok=True)
-    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(obj_dir, "gmm_api.o"), extra),
-             (os.path.join(CSRC, "gmm_probe.hip"), os.path.join(obj_dir, "gmm_probe.o"), extra)]
+    units = [(os.path.join(CSRC, "gmm_api.hip"), os.path.join(obj_dir, "gmm_api.o"), extra)]
     for i in variant_indices():
         units.append((os.path.join(CSRC, "gmm_variant.hip"), os.path.join(obj_dir, f"gmm_variant_{i}.o"),
                       extra + [f"-DGG_VARIANT_INDEX={i}"]))
@@ -123,14 +114,25 @@ def build_binding(force=False):
     return EXT_LIB
 
 
+BENCH_PROBE_SRC = os.path.join(ROOT, "bench_mfma_probe.hip")
+BENCH_PROBE_LIB = os.path.join(ROOT, "libbench_mfma_probe.so")
+
+
+def build_bench_probe(force=False):
+    """bench.py's helper: the rate of the bf16 matrix instruction alone (not part of the library)."""
+    if not force and _newer(BENCH_PROBE_LIB, [BENCH_PROBE_SRC]):
+        return BENCH_PROBE_LIB
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _run([hipcc] + HIPCC_FLAGS + ["-shared", BENCH_PROBE_SRC, "-o", BENCH_PROBE_LIB])
+    return BENCH_PROBE_LIB
+
+
 def build_all(force=False):
     build_hip(force)
     build_binding(force)
+    build_bench_probe(force)
     return HIP_LIB, EXT_LIB
 
 
 if __name__ == "__main__":
-    if "--diagnostic" in sys.argv:
-        print(build_hip(force="--force" in sys.argv, diagnostic=sys.argv[sys.argv.index("--diagnostic") + 1]))
-    else:
-        build_all(force="--force" in sys.argv)
+    build_all(force="--force" in sys.argv)

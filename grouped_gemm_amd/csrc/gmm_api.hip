@@ -162,6 +162,63 @@ int check_common(const int64_t* batch_sizes, int64_t num_groups, int64_t tokens,
   return GG_OK;
 }
 
+// Which kernels a call runs on, from its sizes, element type and the operands' alignment.
+struct Route {
+  uintptr_t address_bits;
+  int elem_bytes;
+  bool indexed;        // any row index given
+  bool indexed_fits;   // ... and a and c are within reach of the streaming kernels' 32-bit offsets
+  bool generic;        // the kernels of gmm_generic.hpp
+  int vec;             // their vector width
+  int64_t a_bytes, c_bytes;
+};
+
+Route classify(const gg_gmm_args& g) {
+  Route r;
+  const int64_t hidden_in = g.hidden_in, hidden_out = g.hidden_out, tokens = g.tokens;
+  const bool trans_a = g.trans_a != 0, trans_b = g.trans_b != 0;
+  const bool swiglu = g.epilogue == GG_EPILOGUE_SWIGLU;
+  r.elem_bytes = g.dtype == GG_DTYPE_F8E4M3 || g.dtype == GG_DTYPE_F8E5M2 ? 1 : 2;
+  r.address_bits =
+      reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b) | reinterpret_cast<uintptr_t>(g.c);
+  // The streaming kernels fetch and store rows 16 bytes at a time: two-byte elements, hidden sizes
+  // that are multiples of 8, operands on 16-byte boundaries, rows in place.  Everything else goes
+  // to the kernels of gmm_generic.hpp, VEC elements at a time.
+  r.indexed = g.a_row_index != nullptr || g.b_row_index != nullptr || g.c_row_index != nullptr;
+  r.a_bytes = (g.a_num_rows > 0 ? g.a_num_rows : tokens) * hidden_in * r.elem_bytes;
+  r.c_bytes = (g.c_num_rows > 0 ? g.c_num_rows : tokens) * hidden_out * 2;
+  // with row indices the streaming kernels address a and c through 32-bit byte offsets
+  r.indexed_fits = !trans_a && r.a_bytes < (int64_t)gg::kOutOfRangeIndexed && r.c_bytes < (int64_t)gg::kOutOfRangeIndexed;
+  // (fp8 streams in 16-byte chunks like the rest: 16 elements, along whichever dimension is
+  // contiguous in each operand)
+  const bool f8_streams = r.elem_bytes == 1 && (!swiglu || (trans_b && !r.indexed)) &&
+                          (trans_a ? hidden_in % 16 == 0 && hidden_out % 16 == 0
+                                   : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
+  r.generic = (r.elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
+              (r.address_bits & 15) || (r.indexed && !r.indexed_fits);
+  r.vec = 8;
+  if (r.generic) {
+    while (r.vec > 1 && (hidden_in % r.vec != 0 || hidden_out % r.vec != 0 ||
+                         (r.address_bits & (uintptr_t)(r.vec * 2 - 1))))
+      r.vec >>= 1;
+  }
+  return r;
+}
+
+// Rows of a, b and c in memory, the bounds a row index is held against: an index that names no
+// row is a missing row (zeros on the way in, nothing stored on the way out) on every kernel.
+struct IndexedRows {
+  int64_t a, b, c;
+};
+
+IndexedRows indexed_rows(const gg_gmm_args& g) {
+  IndexedRows r;
+  r.a = g.a_num_rows > 0 ? g.a_num_rows : g.tokens;
+  r.b = g.b_num_rows > 0 ? g.b_num_rows : g.tokens;
+  r.c = g.c_num_rows > 0 ? g.c_num_rows : g.tokens;
+  return r;
+}
+
 // static_scratch: use the device's static scratch array as the workspace (gg_gmm_no_alloc).
 int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   const int64_t num_groups = g.num_groups, tokens = g.tokens;
@@ -180,7 +237,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     return fail(GG_EINVAL, "the SwiGLU epilogue is for the layouts with a row of c per token and a c of the element type");
   if (swiglu && hidden_in * hidden_out >= (int64_t(1) << 28))
     return fail(GG_ELIMIT, "hidden_in * hidden_out must be below 2^28 with the SwiGLU epilogue");
-  if (g.a_num_rows < 0 || g.c_num_rows < 0) return fail(GG_EINVAL, "negative row count");
+  if (g.a_num_rows < 0 || g.b_num_rows < 0 || g.c_num_rows < 0) return fail(GG_EINVAL, "negative row count");
   if (trans_a && g.c_row_index != nullptr)
     return fail(GG_EINVAL, "c_row_index scatters output rows; the trans_a output has none per token");
   if (!trans_a && g.b_row_index != nullptr)
@@ -194,30 +251,13 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   if (hidden_out == 0 || (trans_a ? hidden_in == 0 : tokens == 0)) return GG_OK;
   if (g.c == nullptr) return fail(GG_EINVAL, "c is null");
   if (tokens > 0 && (g.a == nullptr || g.b == nullptr)) return fail(GG_EINVAL, "a or b is null");
-  const uintptr_t address_bits =
-      reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b) | reinterpret_cast<uintptr_t>(g.c);
+  const Route route = classify(g);
+  const uintptr_t address_bits = route.address_bits;
   if (address_bits & (uintptr_t)(elem_bytes - 1) || reinterpret_cast<uintptr_t>(g.c) & (out_f32 ? 3 : 1))
     return fail(GG_ELIMIT, "a, b and c must be aligned to their element size");
-  // The streaming kernels fetch and store rows 16 bytes at a time: two-byte elements, hidden sizes
-  // that are multiples of 8, operands on 16-byte boundaries, rows in place.  Everything else goes
-  // to the kernels of gmm_generic.hpp, VEC elements at a time.
-  const bool indexed = g.a_row_index != nullptr || g.b_row_index != nullptr || g.c_row_index != nullptr;
-  const int64_t a_bytes = (g.a_num_rows > 0 ? g.a_num_rows : tokens) * hidden_in * elem_bytes;
-  const int64_t c_bytes = (g.c_num_rows > 0 ? g.c_num_rows : tokens) * hidden_out * 2;
-  // with row indices the streaming kernels address a and c through 32-bit byte offsets
-  const bool indexed_fits = !trans_a && a_bytes < (int64_t)gg::kOutOfRangeIndexed && c_bytes < (int64_t)gg::kOutOfRangeIndexed;
-  // (fp8 streams in 16-byte chunks like the rest: 16 elements, along whichever dimension is
-  // contiguous in each operand)
-  const bool f8_streams = elem_bytes == 1 && (!swiglu || (trans_b && !indexed)) &&
-                          (trans_a ? hidden_in % 16 == 0 && hidden_out % 16 == 0
-                                   : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
-  const bool generic = (elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
-                       (address_bits & 15) || (indexed && !indexed_fits);
-  int vec = 8;
-  if (generic) {
-    while (vec > 1 && (hidden_in % vec != 0 || hidden_out % vec != 0 || (address_bits & (uintptr_t)(vec * 2 - 1))))
-      vec >>= 1;
-  }
+  const bool indexed = route.indexed, indexed_fits = route.indexed_fits, generic = route.generic;
+  const int64_t a_bytes = route.a_bytes, c_bytes = route.c_bytes;
+  const int vec = route.vec;
 
   // Host-resident sizes are validated here; they travel in the kernel argument block.
   if (!g.batch_sizes_on_device) {
@@ -266,6 +306,9 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   p.status = g.batch_sizes_on_device ? g.size_status : nullptr;
   p.a_bytes = (uint32_t)(indexed_fits ? a_bytes : 0);
   p.c_bytes = (uint32_t)(indexed_fits ? c_bytes : 0);
+  const IndexedRows index_rows = indexed_rows(g);
+  p.a_index_rows = (uint32_t)(indexed_fits ? index_rows.a : 0);
+  p.c_index_rows = (uint32_t)(indexed_fits ? index_rows.c : 0);
   p.group_m = band_height(num_groups, tokens, trans_a);
   static_assert(GG_FLAG_WHOLE_TILES == gg::kFlagWholeTiles && GG_FLAG_ONE_CLASS == gg::kFlagOneClass &&
                 GG_FLAG_ROW_PIECES == gg::kFlagRowPieces, "the header's flags are the kernel's");
@@ -340,6 +383,9 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
       gp.a_rows = g.a_row_index;
       gp.b_rows = g.b_row_index;
       gp.c_rows = g.c_row_index;
+      gp.a_num_rows = index_rows.a;
+      gp.b_num_rows = index_rows.b;
+      gp.c_num_rows = index_rows.c;
       // light workgroups (28 KiB of LDS): two per compute unit
       const int64_t grid = tiles < 2 * info.cus ? tiles : 2 * info.cus;
       GG_HIP(generic_ops(g.dtype)->launch(layout, vec, epilogue, gp, hs, (int)grid, stream));
@@ -379,6 +425,21 @@ int gg_gmm(const gg_gmm_args* args) {
     return fail(GG_EINVAL, "gg_gmm_args.struct_bytes is %u, this library expects %zu", args->struct_bytes,
                 sizeof(gg_gmm_args));
   return gmm_impl(*args);
+}
+
+uint64_t gg_workspace_bytes_for(const gg_gmm_args* args) {
+  if (args == nullptr || args->struct_bytes != sizeof(gg_gmm_args)) return 0;
+  const gg_gmm_args& g = *args;
+  if (g.dtype < GG_DTYPE_BF16 || g.dtype > GG_DTYPE_F8E5M2 || g.hidden_in <= 0 || g.hidden_out <= 0) return 0;
+  const Route r = classify(g);
+  // (the kernels never cut tiles that are combined or scattered on their way out along the depth)
+  if (r.generic || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
+  if (g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ROW_PIECES)) return 0;
+  if (!g.trans_a) {
+    const int64_t slice = r.elem_bytes == 1 ? 2 * gg::BK : gg::BK;   // depth elements per slice
+    if ((g.hidden_in + slice - 1) / slice < 2 * gg::kMinSlicesPerPiece) return 0;
+  }
+  return GG_WORKSPACE_BYTES;
 }
 
 int gg_gmm_no_alloc(const gg_gmm_args* args) {
@@ -451,18 +512,6 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
     }
   }
   return dispatch_dump(short_shape, layout, p, hs, stream);
-}
-
-int gg_debug_mfma_rate(int zero_operands, int launches, void* stream, float* tflops) {
-  if (tflops == nullptr) return fail(GG_EINVAL, "tflops is null");
-  if (launches < 1 || launches > 1000) return fail(GG_EINVAL, "launches must be 1 .. 1000");
-  DeviceInfo info;
-  const int rc = device_info(&info);
-  if (rc != GG_OK) return rc;
-  // (the kernel never writes through this pointer: the static scratch array is merely a valid one)
-  GG_HIP(gg::run_mfma_probe(info.cus, zero_operands != 0, launches, reinterpret_cast<float*>(info.scratch),
-                            static_cast<hipStream_t>(stream), tflops));
-  return GG_OK;
 }
 
 }  // extern "C"

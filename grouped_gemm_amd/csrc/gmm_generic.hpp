@@ -27,6 +27,9 @@ struct GenericParams {
   const int32_t* a_rows;   // row r of `a` as the product sees it is row a_rows[r] in memory, or nullptr
   const int32_t* b_rows;   // the same for b (weight-gradient layout only), or nullptr
   const int32_t* c_rows;   // row r of the output goes to row c_rows[r] of c (not the weight gradient), or nullptr
+  // rows of a, b and c in memory: an index that names no row of its tensor is a missing row (read
+  // as zeros, not stored), as on the streaming kernels
+  int64_t a_num_rows, b_num_rows, c_num_rows;
 };
 
 namespace generic {
@@ -75,6 +78,7 @@ struct TileLoader {
   int k_end;             // the group's depth
   const int32_t* index;  // rows of the strided dimension in memory, or nullptr
   int index_base;        // position of the group's first row in `index`
+  int64_t index_rows;    // rows the indexed tensor has in memory
   int out_cols;          // GATE_UP: output columns of the group
 
   uint32_t regs[PER_THREAD][VEC * ES > 4 ? VEC * ES / 4 : 1];
@@ -105,9 +109,13 @@ struct TileLoader {
       }
 #pragma unroll
       for (int w = 0; w < (VEC * ES > 4 ? VEC * ES / 4 : 1); ++w) regs[n][w] = 0;
-      if (inside && gk < k_end) {   // extents are multiples of VEC: a vector is all in or all out
-        int64_t strided = K_CONTIGUOUS ? gi : gk;
-        if (index != nullptr) strided = index[index_base + strided];
+      bool present = inside && gk < k_end;   // extents are multiples of VEC: a vector is all in or all out
+      int64_t strided = K_CONTIGUOUS ? gi : gk;
+      if (present && index != nullptr) {
+        strided = index[index_base + strided];
+        present = strided >= 0 && strided < index_rows;   // an index that names no row: zeros
+      }
+      if (present) {
         const char* src = base + (strided * ld + (K_CONTIGUOUS ? gk : gi)) * ES;
         constexpr int NB = VEC * ES;
         if constexpr (NB == 1) {
@@ -212,16 +220,19 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
     aload.k_end = ti.depth;
     aload.index = gp.a_rows;
     aload.index_base = group_row;
+    aload.index_rows = gp.a_num_rows;
     // B: NN rows of b[e] are depth rows (columns contiguous); NT rows are output columns (depth
     // contiguous); weight gradient: rows of b are depth rows
     if (LAYOUT == kTN) {
       bload.base = gp.b_rows ? p.b : p.b + ti.g.b_off * ES;
       bload.index = gp.b_rows;
       bload.index_base = group_row;
+      bload.index_rows = gp.b_num_rows;
     } else {
       bload.base = p.b + ti.g.b_off * ES;
       bload.index = nullptr;
       bload.index_base = 0;
+      bload.index_rows = 0;
     }
     bload.ld = LAYOUT == kNT ? ti.g.k : (GATE_UP ? 2 * ti.g.n : ti.g.n);
     bload.i0 = ti.n0, bload.i_end = ti.g.n;
@@ -274,7 +285,10 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
       const int row = ti.m0 + wm * 64 + i * 32 + (lane & 31);
       if (row >= ti.m0 + ti.rows_valid) continue;
       int64_t mem_row = row;
-      if (gp.c_rows) mem_row = gp.c_rows[out_row0 + row];
+      if (gp.c_rows) {
+        mem_row = gp.c_rows[out_row0 + row];
+        if (mem_row < 0 || mem_row >= gp.c_num_rows) continue;   // an index that names no row: not stored
+      }
       char* crow = cbase + mem_row * ti.g.n * CE;
       if constexpr (GATE_UP) {
         // blocks 0 and 1 of the wave hold the gate and the up value of the same 32 output columns

@@ -70,6 +70,8 @@ struct GmmParams {
   const int32_t* c_rows;   // row r of the output goes to row c_rows[r] of c, or nullptr
   uint32_t a_bytes;        // bytes of a and of c in memory, below kOutOfRangeIndexed
   uint32_t c_bytes;
+  uint32_t a_index_rows;   // rows of a and of c in memory: an index that names no row of them is a
+  uint32_t c_index_rows;   // missing row (read as zeros, not stored)
   int32_t* status;         // device word that collects kStatus* bits about the sizes, or nullptr
 };
 
@@ -535,10 +537,10 @@ struct DepthMajor {
     voff0 = (uint32_t)(row * ld + my_chunk * 8) * 2u;
   }
 
-  // GATHER: the tile's row r is row rows[r] of the tensor at `tensor_base` when `rows` is given,
-  // row first_row + r otherwise; rows past rows_valid_ are out of range.
+  // GATHER: the tile's row r is row rows[r] of the tensor at `tensor_base` (of tensor_rows rows)
+  // when `rows` is given, row first_row + r otherwise; rows past rows_valid_ are out of range.
   __device__ __forceinline__ void setup_gather(const char* tensor_base, uint32_t tensor_bytes,
-                                               const int32_t* rows, int first_row, int ld_,
+                                               const int32_t* rows, uint32_t tensor_rows, int first_row, int ld_,
                                                int rows_valid_, int depth_) {
     base = tensor_base;
     ld = ld_;
@@ -555,7 +557,8 @@ struct DepthMajor {
       uint32_t v = kOutOfRangeIndexed;
       if (r < rows_valid_) {
         const uint32_t src = rows != nullptr ? (uint32_t)rows[r] : (uint32_t)(first_row + r);
-        v = (src * (uint32_t)ld_ + (uint32_t)(my_chunk * 8)) * 2u;
+        // (an index that names no row of the tensor, negative ones included: a row of zeros)
+        if (src < tensor_rows) v = (src * (uint32_t)ld_ + (uint32_t)(my_chunk * 8)) * 2u;
       }
       vrow[i] = v;
     }
@@ -955,21 +958,6 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   return ti;
 }
 
-// Diagnostic builds (build.py --diagnostic no_loads | no_mfma), for timing only, results are
-// wrong: GG_DIAGNOSTIC_NO_LOADS leaves out the loads of the operand tiles (what remains: matrix
-// instructions, LDS reads, barriers, epilogue), GG_DIAGNOSTIC_NO_MFMA all but one matrix
-// instruction per step (what remains: the fetch pipeline, the LDS reads and the epilogue).
-#ifdef GG_DIAGNOSTIC_NO_LOADS
-constexpr bool kDiagnosticNoLoads = true;
-#else
-constexpr bool kDiagnosticNoLoads = false;
-#endif
-#ifdef GG_DIAGNOSTIC_NO_MFMA
-constexpr bool kDiagnosticNoMfma = true;
-#else
-constexpr bool kDiagnosticNoMfma = false;
-#endif
-
 // DT: element type of a and b (and of c unless it is the fp32 accumulator).
 // EPI: what happens to a finished tile (kEpi*): stored in the element type; added to an fp32 c
 // (gradient accumulation, weight-gradient layout); or, with gate | up columns in b, combined to
@@ -1068,7 +1056,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     const int depth = fti.depth;
     if constexpr (INDEXED) {
       const int first = fti.g.row0 + fti.m0;
-      aload.setup_gather(p.a, p.a_bytes, p.a_rows != nullptr ? p.a_rows + first : nullptr, first,
+      aload.setup_gather(p.a, p.a_bytes, p.a_rows != nullptr ? p.a_rows + first : nullptr, p.a_index_rows, first,
                          fti.g.k * ES / 2, depth > 0 ? fti.rows_valid : 0, depth * ES / 2);
     } else if constexpr (Cfg::A_DEPTH_MAJOR) {
       aload.setup(p.a + (fti.g.a_off + (int64_t)fti.m0 * fti.g.k) * ES, fti.g.k * ES / 2, fti.rows_valid,
@@ -1100,8 +1088,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   auto fetch_load = [&](auto j_tag, int buf) {
     constexpr int J = decltype(j_tag)::value;
     const char* st = smem + uniform(buf) * Cfg::STAGE_BYTES;
-    if constexpr (kDiagnosticNoLoads) {
-    } else if constexpr (J < ALoad::NI) {
+    if constexpr (J < ALoad::NI) {
       aload.template load<J>(a_slice, st, wave);
     } else {
       bload.template load<J - ALoad::NI>(b_slice, st + Cfg::A_BYTES, wave);
@@ -1224,12 +1211,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
         constexpr int j = m / ML, i = (j % 2 == 0) ? m % ML : ML - 1 - m % ML;
         // operands swapped: the result block is held transposed, so a lane owns four
         // consecutive columns of one output row
-        if constexpr (!kDiagnosticNoMfma || mm == 0) {
-          if constexpr (F8) {
-            acc[i][j] = mfma_32x32x64_f8<DT>(fb[ks & ~1][j], fb[ks | 1][j], fa[ks & ~1][i], fa[ks | 1][i], acc[i][j]);
-          } else {
-            acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
-          }
+        if constexpr (F8) {
+          acc[i][j] = mfma_32x32x64_f8<DT>(fb[ks & ~1][j], fb[ks | 1][j], fa[ks & ~1][i], fa[ks | 1][i], acc[i][j]);
+        } else {
+          acc[i][j] = mfma_32x32x16<DT>(fb[ks][j], fa[ks][i], acc[i][j]);
         }
         constexpr int u0 = READS * mm / STEP_SLOTS, u1 = READS * (mm + 1) / STEP_SLOTS;
         static_for<u1 - u0>([&](auto d) {
@@ -1301,7 +1286,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
           if (row >= ti.rows_valid) return OOR;
           const int r = ti.g.row0 + ti.m0 + row;
           const uint32_t dst = p.c_rows != nullptr ? (uint32_t)p.c_rows[r] : (uint32_t)r;
-          return dst * (uint32_t)ti.g.n * 2u;
+          return dst < p.c_index_rows ? dst * (uint32_t)ti.g.n * 2u : OOR;   // no such row: not stored
         } else {
           return (uint32_t)(row * ti.g.n) * (uint32_t)CE;
         }

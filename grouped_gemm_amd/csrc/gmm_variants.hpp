@@ -37,8 +37,6 @@ struct GenericOps {
   hipError_t (*launch)(int layout, int vec, int epilogue, const GenericParams& gp, const HostSizes& hs,
                        int grid, hipStream_t stream);
 };
-// gmm_probe.hip: the sustained rate of the matrix instruction alone, operands in registers.
-hipError_t run_mfma_probe(int cus, int zeros, int launches, float* sink, hipStream_t stream, float* tflops);
 
 constexpr int kGenericTileM = 128, kGenericTileN = 128;
 constexpr int kNumElementTypes = 4;   // bf16, f16, f8 e4m3, f8 e5m2

@@ -134,7 +134,8 @@ void Validate(const torch::Tensor& a, const torch::Tensor& b, const torch::Tenso
 }
 
 // Workspace for the depth pieces of a call's last round (see gg_gmm): one per device and stream,
-// allocated and zeroed at the first call there and kept for the life of the process.  Calls on one
+// allocated and zeroed at the first call there that can use one (gg_workspace_bytes_for) and kept
+// for the life of the process.  Calls on one
 // stream run one after the other, so they can share it; the kernels leave its counters zero.
 torch::Tensor Workspace(const torch::Device& device, hipStream_t stream) {
   static std::mutex mu;
@@ -169,7 +170,6 @@ void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
   c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
   hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(a.device().index()).stream();
   TORCH_CHECK(gg_init() == GG_OK, "grouped_gemm: ", gg_last_error());
-  torch::Tensor ws = Workspace(a.device(), stream);
   gg_gmm_args g = {};
   g.struct_bytes = sizeof(g);
   g.dtype = DtypeCode(a.scalar_type());
@@ -191,9 +191,14 @@ void Run(const torch::Tensor& a, const torch::Tensor& b, const torch::Tensor& c,
   g.epilogue = gate_up ? GG_EPILOGUE_SWIGLU : GG_EPILOGUE_NONE;
   g.a_num_rows = a.size(0);
   g.c_num_rows = trans_a ? 0 : c.size(0);
-  g.workspace = ws.data_ptr();
-  g.workspace_bytes = (uint64_t)ws.numel();
+  g.b_num_rows = trans_a ? (int32_t)b.size(0) : 0;
   g.flags = (int32_t)flags;
+  // a workspace only for calls that can cut tiles along the depth (deep products, weight gradients)
+  if (gg_workspace_bytes_for(&g) > 0) {
+    torch::Tensor ws = Workspace(a.device(), stream);
+    g.workspace = ws.data_ptr();
+    g.workspace_bytes = (uint64_t)ws.numel();
+  }
   g.stream = static_cast<void*>(stream);
   if (sizes.is_cuda()) g.size_status = SizeStatusWord(a.device()).data_ptr<int32_t>();
   const int rc = gg_gmm(&g);
@@ -284,19 +289,6 @@ torch::Tensor DebugSchedule(torch::Tensor batch_sizes, int64_t tokens, int64_t h
   return out;
 }
 
-// TFLOP/s the device sustains on the bf16 matrix instruction alone, operands in registers
-// (see gg_debug_mfma_rate); waits for the device.
-double MfmaRate(torch::Device device, bool zero_operands, int64_t launches) {
-  TORCH_CHECK(device.is_cuda(), "grouped_gemm: the probe runs on a GPU");
-  c10::hip::HIPGuardMasqueradingAsCUDA guard(device);
-  if (!device.has_index()) device = torch::Device(device.type(), c10::hip::current_device());
-  hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(device.index()).stream();
-  float tflops = 0.0f;
-  const int rc = gg_debug_mfma_rate(zero_operands ? 1 : 0, (int)launches, static_cast<void*>(stream), &tflops);
-  TORCH_CHECK(rc == GG_OK, "grouped_gemm: ", gg_last_error());
-  return tflops;
-}
-
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("gmm", &GroupedGemm, "Grouped GEMM.");
   m.def("validate",
@@ -319,8 +311,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,
         "c (fp32) += per expert a_e^T @ b_e.");
   m.def("debug_schedule", &DebugSchedule, "Per-group table derived by the on-device scheduler.");
-  m.def("mfma_rate", &MfmaRate, "TFLOP/s of the bf16 matrix instruction alone, operands in registers.",
-        py::arg("device"), py::arg("zero_operands") = false, py::arg("launches") = 5);
   m.attr("max_groups_per_launch") = GG_MAX_GROUPS_PER_LAUNCH;
   m.attr("sched_cols") = GG_SCHED_COLS;
 }

@@ -9,8 +9,9 @@
  * gg_gmm_bf16.
  *
  * All functions return 0 on success and a negative GG_E* code on failure;
- * gg_last_error() then holds a message for the calling thread.  No entry point
- * synchronises the device or allocates device memory.
+ * gg_last_error() then holds a message for the calling thread
+ * (gg_workspace_bytes_for returns a size).  No entry point synchronises the device or
+ * allocates device memory.
  */
 #ifndef GROUPED_GEMM_HIP_H_
 #define GROUPED_GEMM_HIP_H_
@@ -142,10 +143,12 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  *   b_row_index   the same for the rows of b, trans_a layout only.
  *   c_row_index   int32[tokens] on the device, or NULL: row r of the output is stored to row
  *                 c_row_index[r] of c (a scatter fused into the store; not with trans_a).  Rows of
- *                 c that no index names are not touched.  Indices are not checked: each must
- *                 name a row that exists, and c_row_index must not name a row twice.
- *   a_num_rows, c_num_rows
- *                 Rows of a and of c in memory when a row index redirects them (0: `tokens`).
+ *                 c that no index names are not touched.  c_row_index must not name a row twice.
+ *                 An index that names no row of its tensor (negative, or past the row count
+ *                 below) is a missing row on every kernel: zeros on the way in, nothing stored
+ *                 on the way out; no such index can make a kernel touch memory outside a, b, c.
+ *   a_num_rows, b_num_rows, c_num_rows
+ *                 Rows of a, b and c in memory when a row index redirects them (0: `tokens`).
  *                 With two-byte elements, aligned operands and a and c below 4 GiB the NN and NT
  *                 layouts run indexed on the streaming kernels; otherwise, and with trans_a, on
  *                 the general ones.
@@ -200,11 +203,22 @@ typedef struct gg_gmm_args {
   int64_t a_num_rows;
   int64_t c_num_rows;
   int32_t epilogue;
-  int32_t reserved1;
+  int32_t b_num_rows;
   int32_t* size_status;
 } gg_gmm_args;
 
 int gg_gmm(const gg_gmm_args* args);
+
+/*
+ * Bytes of workspace the call described by `args` can make use of: 0 when no launch of it ever
+ * cuts tiles along the depth (general kernels, row indices, the SwiGLU epilogue, or a product too
+ * shallow for depth pieces to pay: fewer than 96 depth slices of 64 two-byte or 128 one-byte
+ * elements outside the trans_a layout), GG_WORKSPACE_BYTES otherwise.  Looks at the sizes, flags
+ * and pointers' alignment only; args->workspace is ignored.  A caller that keeps workspaces
+ * (one per stream) need not allocate one for calls this returns 0 for.  No counterpart in the
+ * reference, which asks CUTLASS for its workspace size per call (csrc/grouped_gemm.cu:347-349).
+ */
+uint64_t gg_workspace_bytes_for(const gg_gmm_args* args);
 
 /*
  * gg_gmm for callers that cannot allocate and have no workspace to bring: code under HIP graph
@@ -236,16 +250,6 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device,
                       int64_t num_groups, int64_t tokens, int64_t hidden_in,
                       int64_t hidden_out, int trans_a, int trans_b, int64_t* table_out,
                       void* stream);
-
-/*
- * A probe, no counterpart in the reference: the rate (TFLOP/s, through `tflops`) at which the
- * device sustains the bf16 matrix instruction the kernels are built on, with operands in
- * registers and no memory traffic; on operands with the bit statistics of randn * 0.02 data
- * (zero_operands = 0) or on zeros.  The first is the ceiling the device's power limit sets for any
- * bf16 GEMM on such data; benchmarks print it next to the GEMM's rate.  Runs `launches` + 1
- * launches of about 2 ms on `stream` and waits for them.
- */
-int gg_debug_mfma_rate(int zero_operands, int launches, void* stream, float* tflops);
 
 /* Output tile (rows, columns) and depth slice the kernel uses for a call with these arguments
  * (calls whose groups average few rows get a shorter tile); for reports and for checking the

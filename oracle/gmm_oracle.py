@@ -12,6 +12,11 @@ Contents
                       up-cast first, which gives the fp32-accumulated result the
                       tolerance is stated against.
   swiglu_loop         the gated activation silu(a @ gate) * (a @ up) on top of that loop.
+  swiglu_parts / swiglu_tolerance
+                      the same in float64 together with its two pre-activations, and the
+                      acceptance rule for it when the pre-activations are large (deep products of
+                      unscaled operands): the output tolerance plus what an fp32 accumulation
+                      error of a pre-activation becomes once the other one multiplies it.
   gmm_c               same result from the plain-C triple loop in gg_oracle.c
                       (small shapes only).
   table_walk / table_closed / table_numpy
@@ -134,6 +139,46 @@ def swiglu_loop(a, b, batch_sizes, trans_b=False, dtype=torch.float32):
     gate = gmm_loop(a, gate_w.contiguous(), batch_sizes, trans_b=trans_b, dtype=dtype)
     up = gmm_loop(a, up_w.contiguous(), batch_sizes, trans_b=trans_b, dtype=dtype)
     return gate / (1.0 + torch.exp(-gate)) * up
+
+
+def swiglu_parts(a, b, batch_sizes, trans_b=False):
+    """(out, gate, up) in float64: the two pre-activations a_e @ gate_e and a_e @ up_e from the
+    per-expert loop above and out = silu(gate) * up."""
+    half = (b.shape[1] if trans_b else b.shape[2]) // 2
+    gate_w = b[:, :half] if trans_b else b[:, :, :half]
+    up_w = b[:, half:] if trans_b else b[:, :, half:]
+    gate = gmm_loop(a, gate_w.contiguous(), batch_sizes, trans_b=trans_b, dtype=torch.float64)
+    up = gmm_loop(a, up_w.contiguous(), batch_sizes, trans_b=trans_b, dtype=torch.float64)
+    return gate * torch.sigmoid(gate) * up, gate, up
+
+
+# A pre-activation summed in fp32 over K products carries an error of about 2^-24 times the size of
+# its partial sums per addition.  The matrix instruction adds 16 products at a time, so there are
+# K / 16 additions; with errors that do not line up their sum grows like the square root of that
+# count.  The factor in front covers the largest of ~10^7 such sums and partial sums a few times
+# the typical pre-activation (measured on deep unscaled products: a tenth of this bound).
+PREACT_ERROR_FACTOR = 10.0
+
+
+def swiglu_tolerance(want, gate, up, hidden_in, rtol=RTOL, atol=ATOL):
+    """Per-element tolerance for silu(gate) * up computed from fp32-accumulated pre-activations.
+
+    out = silu(g) * u has d out = u * silu'(g) * dg + silu(g) * du: where one pre-activation is
+    near zero and the other is large (|u| of a few hundred with unscaled operands and a depth of
+    thousands), the output is small and an fp32 summation error dg of 1e-4 moves it by more than
+    any tolerance proportional to the output.  No fp32-accumulating implementation can meet
+    atol + rtol * |want| there (the per-expert loop in fp32 does not either), so the rule adds
+    exactly that term: (|u * silu'(g)| + |silu(g)|) * delta with
+    delta = PREACT_ERROR_FACTOR * 2^-24 * sqrt(hidden_in / 16) * rms(pre-activations),
+    silu'(g) = s * (1 + g * (1 - s)), s = sigmoid(g).  For pre-activations of unit size the added
+    term is far below atol and the rule is the plain one."""
+    want, gate, up = want.double(), gate.double(), up.double()
+    sig = torch.sigmoid(gate)
+    dsilu = sig * (1.0 + gate * (1.0 - sig))
+    scale = float(torch.cat([gate.flatten(), up.flatten()]).pow(2).mean().sqrt()) if gate.numel() else 0.0
+    delta = PREACT_ERROR_FACTOR * 2.0 ** -24 * (max(hidden_in, 16) / 16.0) ** 0.5 * scale
+    plain = atol_for(want.float(), atol) + rtol * want.abs()
+    return plain + ((up * dsilu).abs() + (gate * sig).abs()) * delta
 
 
 def accumulate_weight_gradient_loop(a, b, batch_sizes, c0, dtype=torch.float64):

@@ -202,7 +202,7 @@ class _Args(ctypes.Structure):
                 ("flags", ctypes.c_int32), ("reserved0", ctypes.c_int32), ("stream", ctypes.c_void_p),
                 ("a_row_index", ctypes.c_void_p), ("b_row_index", ctypes.c_void_p), ("c_row_index", ctypes.c_void_p),
                 ("a_num_rows", ctypes.c_int64), ("c_num_rows", ctypes.c_int64),
-                ("epilogue", ctypes.c_int32), ("reserved1", ctypes.c_int32), ("size_status", ctypes.c_void_p)]
+                ("epilogue", ctypes.c_int32), ("b_num_rows", ctypes.c_int32), ("size_status", ctypes.c_void_p)]
 
 
 def test_general_entry_point_argument_errors_need_no_device():
@@ -234,8 +234,52 @@ def test_general_entry_point_argument_errors_need_no_device():
     rc, msg = call(b_row_index=64)
     assert rc == -1 and b"b_row_index" in msg
     assert call(a_num_rows=-1)[0] == -1
+    assert call(b_num_rows=-1)[0] == -1
+    assert call(c_num_rows=-1)[0] == -1
     rc, msg = call(c=12288 + 1)
     assert rc == -2 and b"element size" in msg
+
+
+def test_workspace_bytes_for_needs_no_device():
+    """gg_workspace_bytes_for: nothing for calls that can never cut tiles along the depth, the
+    full workspace for deep products and weight gradients."""
+    lib = ctypes.CDLL(HIP_LIB)
+    lib.gg_workspace_bytes_for.argtypes = [ctypes.c_void_p]
+    lib.gg_workspace_bytes_for.restype = ctypes.c_uint64
+    full = 4096 + 256 * 256 * 256 * 4
+
+    def want(**kw):
+        g = _Args()
+        g.struct_bytes = ctypes.sizeof(_Args)
+        g.a, g.b, g.c = 4096, 8192, 12288
+        g.num_groups, g.tokens, g.hidden_in, g.hidden_out = 8, 32768, 4096, 14336
+        for k, v in kw.items():
+            setattr(g, k, v)
+        return lib.gg_workspace_bytes_for(ctypes.byref(g))
+
+    assert lib.gg_workspace_bytes_for(None) == 0
+    assert want(struct_bytes=4) == 0
+    assert want() == 0                                     # 64 depth slices: too shallow
+    assert want(hidden_in=14336, hidden_out=4096) == full  # 224 slices
+    assert want(hidden_in=6144) == full and want(hidden_in=6080) == 0
+    assert want(trans_a=1) == full                         # the depth is the group's rows
+    assert want(trans_a=1, hidden_in=4097) == 0            # general kernels
+    assert want(trans_a=1, a=4096 + 2) == 0                # off the 16-byte boundary
+    assert want(hidden_in=14336, a_row_index=64) == 0      # scattered or gathered tiles stay whole
+    assert want(hidden_in=14336, hidden_out=2048, epilogue=1) == 0
+    assert want(hidden_in=14336, flags=1) == 0 and want(hidden_in=14336, flags=4) == 0
+    assert want(dtype=2, hidden_in=12288) == full and want(dtype=2, hidden_in=12160) == 0
+
+
+def test_row_index_bounds_reach_every_kernel():
+    """The C ABI hands the row counts that bound a row index to the general kernels as it does to
+    the streaming ones (checked in the sources: no GPU test feeds bad indices on purpose)."""
+    api = open(os.path.join(ROOT, "grouped_gemm_amd", "csrc", "gmm_api.hip")).read()
+    for field in ("gp.a_num_rows = index_rows.a", "gp.b_num_rows = index_rows.b", "gp.c_num_rows = index_rows.c",
+                  "p.a_index_rows =", "p.c_index_rows ="):
+        assert field in api, field
+    generic = open(os.path.join(ROOT, "grouped_gemm_amd", "csrc", "gmm_generic.hpp")).read()
+    assert "strided < index_rows" in generic and "mem_row >= gp.c_num_rows" in generic
 
 
 # ----------------------------------------------------------------- workloads

@@ -109,6 +109,49 @@ def test_swiglu_loop_known_values(oracle):
     torch.testing.assert_close(nn, want, rtol=1e-6, atol=1e-6)
 
 
+def test_swiglu_parts_and_tolerance_rule(oracle):
+    import math
+    # swiglu_parts: the float64 form agrees with the closed form at hand-fixed points and with the
+    # fp32 loop on random data
+    a = torch.ones(1, 1, dtype=torch.bfloat16)
+    out, gate, up = oracle.swiglu_parts(a, torch.tensor([[[2.0, 3.0]]], dtype=torch.bfloat16), torch.tensor([1]))
+    assert out.dtype == torch.float64 and float(gate) == 2.0 and float(up) == 3.0
+    assert abs(float(out) - 6.0 / (1.0 + math.exp(-2.0))) < 1e-12
+    g = torch.Generator().manual_seed(4)
+    a2 = torch.randn(9, 24, generator=g).to(torch.bfloat16)
+    b2 = torch.randn(3, 24, 10, generator=g).to(torch.bfloat16)
+    bs = torch.tensor([4, 0, 5])
+    for tb in (False, True):
+        bb = b2.transpose(1, 2).contiguous() if tb else b2
+        out, gate, up = oracle.swiglu_parts(a2, bb, bs, trans_b=tb)
+        torch.testing.assert_close(out.float(), oracle.swiglu_loop(a2, bb, bs, trans_b=tb), rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(gate.float(), oracle.gmm_loop(a2, b2[:, :, :5].contiguous(), bs), rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(up.float(), oracle.gmm_loop(a2, b2[:, :, 5:].contiguous(), bs), rtol=1e-6, atol=1e-6)
+    # the derivative the rule uses, against central differences of x / (1 + exp(-x)) in float64
+    silu = lambda x: x / (1.0 + math.exp(-x))
+    for x in (-30.0, -3.0, -0.5, 0.0, 0.7, 4.0, 25.0):
+        sgm = 1.0 / (1.0 + math.exp(-x))
+        assert abs(sgm * (1.0 + x * (1.0 - sgm)) - (silu(x + 1e-6) - silu(x - 1e-6)) / 2e-6) < 1e-8
+    # the rule itself at a point worked out by hand: gate = 0, up = 200 (silu'(0) = 1/2, silu(0) = 0),
+    # depth 8192 (sqrt(8192 / 16) = 22.627), pre-activation rms = sqrt((0 + 200^2) / 2) = 141.42:
+    # delta = 10 * 2^-24 * 22.627 * 141.42 = 1.9073e-3, added term = 200 * 0.5 * delta = 0.19073
+    want = torch.zeros(1, 1, dtype=torch.float64)
+    tol = oracle.swiglu_tolerance(want, torch.zeros(1, 1), torch.full((1, 1), 200.0), 8192)
+    assert abs(float(tol) - (0.0 + 0.19073)) < 2e-5, float(tol)    # rms(want) = 0: no absolute term
+    # unit-size pre-activations: the added term is far below the plain tolerance
+    gate, up = torch.randn(64, 64, generator=g).double(), torch.randn(64, 64, generator=g).double()
+    want = gate * torch.sigmoid(gate) * up
+    tol = oracle.swiglu_tolerance(want, gate, up, 512)
+    plain = oracle.atol_for(want.float()) + oracle.RTOL * want.abs()
+    assert float((tol - plain).max()) < 0.01 * oracle.atol_for(want.float())
+    # and a dropped product (one term of size 1 missing from a pre-activation of a deep sum) is
+    # still far outside it: d out = up * silu'(gate) * 1
+    gate, up = torch.full((1, 1), 0.3, dtype=torch.float64), torch.full((1, 1), 150.0, dtype=torch.float64)
+    want = gate * torch.sigmoid(gate) * up
+    wrong = (gate - 1.0) * torch.sigmoid(gate - 1.0) * up
+    assert float((wrong - want).abs()) > 50 * float(oracle.swiglu_tolerance(want, gate, up, 8192))
+
+
 def test_float8_decode_known_values():
     # the oracle for fp8 operands is the per-expert loop on torch's fp32 decode of the bytes; pin the
     # decode on values fixed by the OCP formats (1.0, the largest finite value, the smallest
