@@ -124,7 +124,7 @@ WORKLOAD_NAMES = {
 }
 
 
-def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0):
+def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0, only=None):
     """Times the grouped GEMMs of one configuration; returns (workload, names, layout, ms_per_step,
     per-launch samples in ms)."""
     import torch
@@ -149,7 +149,7 @@ def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0):
         "agrad": lambda: gmm(w.grad, w.b, trans_b=not w.trans_b),
         "bgrad": lambda: gmm(lhs, rhs, trans_a=True),
     }
-    names = [n for n in ("fwd", "agrad", "bgrad") if n in w.gemms]
+    names = [n for n in ("fwd", "agrad", "bgrad") if n in (only or w.gemms)]
     if accumulate:
         main_grad = torch.zeros(w.batch_sizes.numel(), lhs.shape[1], rhs.shape[1], device="cuda")
         calls["bgrad"] = lambda: backend.accumulate_weight_gradient(lhs, rhs, sizes_dev, main_grad)
@@ -274,10 +274,14 @@ def other_paths(steps=7, warmup=4):
     au, bu = w.a[:, :hin].contiguous(), w.b[:, :hin, :hout].contiguous()
     res[f"hidden sizes {hin} x {hout} (zero-padded copies, streaming kernel)"] = timed(
         lambda: backend.gmm(au, bu, sd), reps=2, f=2 * t * hin * hout)
-    backend.PAD_ODD_SIZES = False
-    res[f"hidden sizes {hin} x {hout} (general kernels)"] = timed(lambda: backend.gmm(au, bu, sd), reps=2,
-                                                                 f=2 * t * hin * hout)
-    backend.PAD_ODD_SIZES = True
+    cu = torch.empty(t, hout, dtype=torch.bfloat16, device="cuda")
+    res[f"hidden sizes {hin} x {hout} (general kernels, the extension called directly)"] = timed(
+        lambda: backend.backend.gmm(au, bu, cu, sd, False, False), reps=2, f=2 * t * hin * hout)
+    del au, bu
+    # b stored transposed: only the depth has to be a multiple of 8, an even width streams as it is
+    bt = w.b[:, :, :hout].transpose(1, 2).contiguous()
+    res[f"hidden sizes {w.hidden_in} x {hout}, b stored transposed (streaming kernel, no copies)"] = timed(
+        lambda: backend.gmm(w.a, bt, sd, trans_b=True, c=cu), f=2 * t * w.hidden_in * hout)
     return res
 
 
@@ -287,6 +291,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration (2 = Mixtral w1)")
+    ap.add_argument("--only", default=None, help="time only these GEMMs of the configuration: a comma-separated "
+                    "subset of fwd,agrad,bgrad (bgrad also for a configuration that lists only its forward GEMM)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the short runs of the other configurations that the default run appends")
@@ -323,11 +329,12 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copied_bytes": args.copy_bytes, "times": 5}))
         return
+    only = tuple(args.only.split(",")) if args.only else None
     w, names, layout, ms_per_step, samples = run_workload(args.config, args.steps, args.warmup,
-                                                          args.accumulate, args.zeros, args.flags)
+                                                          args.accumulate, args.zeros, args.flags, only)
     value, roofline, slowest, kernel_ms = summarize(w, names, layout, ms_per_step, samples, args.accumulate)
     flops_gemm = w.flops_per_gemm()
-    traffic = MEASURED_TRAFFIC.get(args.config, {}).get(slowest) if not (args.zeros or args.accumulate or args.flags) else None
+    traffic = MEASURED_TRAFFIC.get(args.config, {}).get(slowest) if not (args.zeros or args.accumulate or args.flags or only) else None
     roofline["traffic"] = round(traffic["bytes"]) if traffic else None
     roofline["traffic_source"] = traffic["source"] if traffic else None
     metric, what = WORKLOAD_NAMES[args.config]
@@ -404,16 +411,20 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)
     # The other measured configurations, shortly, so that one default run shows all of them.
-    default_run = not (args.no_other_configs or args.zeros or args.flags or args.accumulate or args.vendor_loop)
+    default_run = not (args.no_other_configs or args.zeros or args.flags or args.accumulate or args.vendor_loop or only)
     if default_run and args.config == 2:
         del w
         others = {}
-        for cfg, acc in ((3, False), (4, False), (4, True), (5, False)):
+        # (configs[2] is a forward GEMM; its weight gradient, with Zipf depths and empty groups, is
+        # timed beside it as the ragged case of the trans_a layout)
+        for cfg, acc, only in ((3, False, None), (3, False, ("bgrad",)), (4, False, None), (4, True, None),
+                               (5, False, None)):
             torch.cuda.empty_cache()
-            res = run_workload(cfg, min(args.steps, 10), min(args.warmup, 3), accumulate=acc)
+            res = run_workload(cfg, min(args.steps, 10), min(args.warmup, 3), accumulate=acc, only=only)
             v, roof, _, _ = summarize(*res, accumulate=acc)
-            others[f"configs[{cfg - 1}]" + (" accumulate" if acc else "")] = {
-                "workload": WORKLOAD_NAMES[cfg][1] if not acc else "weight gradient added to an fp32 output",
+            others[f"configs[{cfg - 1}]" + (" accumulate" if acc else "") + (" weight gradient" if only else "")] = {
+                "workload": ("weight-gradient grouped GEMM of the same workload" if only else
+                             WORKLOAD_NAMES[cfg][1] if not acc else "weight gradient added to an fp32 output"),
                 "experts": res[0].batch_sizes.numel(), "rows": res[0].tokens,
                 "hidden": f"{res[0].hidden_in}x{res[0].hidden_out}", "steps": min(args.steps, 10),
                 "ms_per_step": round(res[3], 4), "TFLOP/s": round(v, 2),

@@ -168,6 +168,7 @@ struct Route {
   int elem_bytes;
   bool indexed;        // any row index given
   bool indexed_fits;   // ... and a and c are within reach of the streaming kernels' 32-bit offsets
+  bool ragged_width;   // streaming kernel, b stored transposed, width even but not a multiple of 8
   bool generic;        // the kernels of gmm_generic.hpp
   int vec;             // their vector width
   int64_t a_bytes, c_bytes;
@@ -194,8 +195,17 @@ Route classify(const gg_gmm_args& g) {
   const bool f8_streams = r.elem_bytes == 1 && (!swiglu || (trans_b && !r.indexed)) &&
                           (trans_a ? hidden_in % 16 == 0 && hidden_out % 16 == 0
                                    : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
-  r.generic = (r.elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
-              (r.address_bits & 15) || (r.indexed && !r.indexed_fits);
+  // b stored transposed: rows of a and of b run along the depth, so only the depth has to be a
+  // multiple of 8; an even width that is not leaves rows of c on 4-byte boundaries, which the
+  // store epilogue of the streaming kernel handles (two-byte elements, c of the same type)
+  r.ragged_width = r.elem_bytes == 2 && trans_b && !trans_a && !swiglu && !g.accumulate_f32 &&
+                   hidden_in % 8 == 0 && hidden_out % 8 != 0 && hidden_out % 2 == 0 &&
+                   ((reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b)) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(g.c) & 3) == 0;
+  r.generic = !r.ragged_width &&
+              ((r.elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
+               (r.address_bits & 15));
+  r.generic = r.generic || (r.indexed && !r.indexed_fits);
   r.vec = 8;
   if (r.generic) {
     while (r.vec > 1 && (hidden_in % r.vec != 0 || hidden_out % r.vec != 0 ||
@@ -324,12 +334,14 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     p.ws_slots = (int32_t)(((uint64_t)GG_WORKSPACE_BYTES - gg::kWsCounterBytes) /
                            ((uint64_t)bm * bn * (swiglu ? 2 : 1) * 4));
     if (p.ws_slots > 1024) p.ws_slots = 1024;
+    // (the fix-up of depth pieces stores 4 columns at a time: whole tiles and row pieces only)
+    if (route.ragged_width) p.ws_slots = 0;
     // Every call on this device shares the array and finds what the last call left: the arrival
     // counters must start at zero (a fill kernel, not a memset: callers may be capturing a graph).
     hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(gg::kWsCounterBytes / 4), 0, stream,
                        reinterpret_cast<int*>(info.scratch));
     GG_HIP(hipGetLastError());
-  } else if (g.workspace != nullptr && !generic) {
+  } else if (g.workspace != nullptr && !generic && !route.ragged_width) {
     if (reinterpret_cast<uintptr_t>(g.workspace) & 255)
       return fail(GG_ELIMIT, "the workspace must be 256-byte aligned");
     const uint64_t slot_bytes = (uint64_t)bm * bn * (swiglu ? 2 : 1) * 4;
@@ -433,7 +445,7 @@ uint64_t gg_workspace_bytes_for(const gg_gmm_args* args) {
   if (g.dtype < GG_DTYPE_BF16 || g.dtype > GG_DTYPE_F8E5M2 || g.hidden_in <= 0 || g.hidden_out <= 0) return 0;
   const Route r = classify(g);
   // (the kernels never cut tiles that are combined or scattered on their way out along the depth)
-  if (r.generic || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
+  if (r.generic || r.ragged_width || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
   if (g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ROW_PIECES)) return 0;
   if (!g.trans_a) {
     const int64_t slice = r.elem_bytes == 1 ? 2 * gg::BK : gg::BK;   // depth elements per slice

@@ -191,6 +191,10 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
   __shared__ __attribute__((aligned(16))) char tile_b[BN * PITCH];
   build_schedule<LAYOUT, BM, BNS>(&sched, p, hs);
   __syncthreads();
+  if constexpr (LAYOUT == kTN) {
+    order_groups_by_depth(&sched, p.num_groups);
+    __syncthreads();
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;

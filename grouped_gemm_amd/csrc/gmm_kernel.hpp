@@ -164,6 +164,12 @@ struct Sched {
   int32_t tile_start[kMaxGroups + 1];  // exclusive prefix sum of the first class's tiles
   int32_t runt_start[kMaxGroups + 1];  // exclusive prefix sum of the runt rows' tiles
   int32_t arrived;                     // broadcast slot for the arrival count of a depth piece
+  // Weight-gradient layout only: the groups by descending depth (order[q] is the group whose tiles
+  // are handed out q-th).  Every group has the same number of tiles there and a tile's cost is its
+  // group's depth, so the deepest groups go first and the shallow ones fill the end of the launch:
+  // what the reference's sort by k does for its scheduler (csrc/grouped_gemm.cu:193-207,
+  // csrc/fill_arguments.cuh:80-81).  Results do not depend on it.
+  int16_t order[kMaxGroups];
 };
 
 constexpr uint32_t kOutOfRange = 0x80000000u;  // beyond any descriptor size used here
@@ -410,6 +416,22 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
   }
 }
 
+// Run by every thread of the workgroup after build_schedule and a barrier (weight-gradient layout
+// only); the caller puts a barrier behind it.  Stable: groups of equal depth keep their order.
+// Thread t ranks groups t, t + blockDim, ...: a group's position is the number of groups that go
+// before it.
+__device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups) {
+  for (int e = threadIdx.x; e < num_groups; e += blockDim.x) {
+    const int mine = s->rows[e];
+    int before = 0;
+    for (int j = 0; j < num_groups; ++j) {
+      const int other = s->rows[j];   // (the same address in every lane: a broadcast read)
+      before += (other > mine || (other == mine && j < e)) ? 1 : 0;
+    }
+    s->order[before] = (int16_t)e;
+  }
+}
+
 // Element offsets of a group's A, B and C blocks, the quantities of the reference's
 // problem table (csrc/fill_arguments.cuh:72-76) in int64.  The kernel addresses memory
 // through these and the schedule dump prints these.
@@ -464,6 +486,10 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSize
   __shared__ Sched s;
   build_schedule<LAYOUT, BM, BN>(&s, p, hs);
   __syncthreads();
+  if (LAYOUT == kTN) {
+    order_groups_by_depth(&s, p.num_groups);
+    __syncthreads();
+  }
   for (int e = threadIdx.x; e < p.num_groups; e += 64) {
     const GroupGeom g = group_geometry<LAYOUT>(p, p.first_group + e, s.row_start[e], s.rows[e]);
     const GroupTiles gt = group_tiles<LAYOUT, BM, BN>(s.rows[e], p.hidden_in, p.hidden_out, p.flags);
@@ -477,7 +503,12 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSize
     row[6] = g.a_off;
     row[7] = g.b_off;
     row[8] = g.c_off;
-    row[9] = s.tile_start[e];
+    int position = e;   // where the group's tiles stand in the order they are handed out
+    if (LAYOUT == kTN) {
+      for (int q = 0; q < p.num_groups; ++q)
+        if (s.order[q] == e) position = q;
+    }
+    row[9] = s.tile_start[position];
     row[10] = gt.tiles_m * gt.tiles_n;
     row[11] = s.rows[e];
     row[12] = s.tile_start[p.num_groups] + s.runt_start[e];
@@ -910,7 +941,9 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
     while (t >= uniform(sched->runt_start[cur.e + 1])) ++cur.e;
     u = t - uniform(sched->runt_start[cur.e]);
   }
-  const int e = cur.e;
+  // (weight-gradient layout: the cursor walks positions of the descending-depth order; all groups
+  // have the same number of tiles there, so the tile prefix sums serve positions as they are)
+  const int e = LAYOUT == kTN ? uniform((int)sched->order[cur.e]) : cur.e;
   // read through the first lane: everything derived from these stays in scalar registers
   const int rows = uniform(sched->rows[e]);
   ti.g = group_geometry<LAYOUT>(p, p.first_group + e, uniform(sched->row_start[e]), rows);
@@ -999,6 +1032,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   Sched* sched = reinterpret_cast<Sched*>(smem + Cfg::SCHED_OFFSET);
   build_schedule<LAYOUT, BM, BNS>(sched, p, hs);
   __syncthreads();
+  if constexpr (LAYOUT == kTN) {
+    order_groups_by_depth(sched, p.num_groups);
+    __syncthreads();
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
@@ -1406,6 +1443,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
         constexpr int PITCH = Cfg::EPILOGUE_PITCH;
         const int in_row = lane & 31, in_half = lane >> 5;
         const int out_row = lane >> 3, out_chunk = lane & 7;
+        // NT layout: an even width that is not a multiple of 8 (rows of c then start on 4-byte
+        // boundaries only, and the last 16-byte chunk of a row holds 2, 4 or 6 columns)
+        const bool ragged_width = LAYOUT == kNT && uniform(ti.g.n & 7) != 0;
 #pragma unroll
         for (int i = 0; i < ML; ++i) {
           uint32_t row_off[4];
@@ -1423,7 +1463,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
             for (int r = 0; r < 4; ++r) {
               const u32x4 v = *reinterpret_cast<const u32x4*>(strip + (r * 8 + out_row) * PITCH + out_chunk * 16);
               const int col = ti.n0 + wn * Cfg::WTN + jp * 64 + out_chunk * 8;
-              __builtin_amdgcn_raw_buffer_store_b128(v, rc, at(row_off[r], col), 0, kStoreStreaming);
+              // (whole chunks only: for widths that are multiples of 8 the same as col < n)
+              __builtin_amdgcn_raw_buffer_store_b128(v, rc, col + 8 <= ti.g.n ? at(row_off[r], col) : OOR, 0,
+                                                     kStoreStreaming);
+              if constexpr (LAYOUT == kNT) {
+                if (ragged_width) {
+                  const int valid = ti.g.n - col;   // columns of this lane's chunk that exist
+                  const uint32_t off = at(row_off[r], col);
+                  if (valid > 0 && valid < 8 && off != OOR) {
+                    if (valid & 4) __builtin_amdgcn_raw_buffer_store_b64(u32x2{v[0], v[1]}, rc, off, 0, kStoreStreaming);
+                    if (valid & 2)
+                      __builtin_amdgcn_raw_buffer_store_b32((valid & 4) ? v[2] : v[0], rc, off + ((valid & 4) ? 8u : 0u), 0,
+                                                            kStoreStreaming);
+                  }
+                }
+              }
             }
             // keep the conversion of one strip from being hoisted over the stores of the
             // previous one: few accumulators are live in vector registers at a time

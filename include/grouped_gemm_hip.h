@@ -232,6 +232,10 @@ uint64_t gg_workspace_bytes_for(const gg_gmm_args* args);
  * (different streams, different threads) race on it and must be serialised by the caller.
  * The array holds one partial tile per workgroup of a launch of up to 256 workgroups: a device
  * with more compute units is rejected (GG_ELIMIT), as is a non-NULL workspace (GG_EINVAL).
+ * gg_init (or any earlier call of the library on that device) must come first where the call
+ * itself must not allocate or is being captured: the first call on a device loads the kernels'
+ * code object, raises their LDS limits and looks the array's address up.  Without depth pieces to
+ * cut (gg_workspace_bytes_for returns 0) the result equals gg_gmm's with workspace = NULL.
  */
 int gg_gmm_no_alloc(const gg_gmm_args* args);
 

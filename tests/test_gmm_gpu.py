@@ -292,6 +292,30 @@ def test_config3_ragged_full_size(ops, oracle):
         check(ops.backend.gmm(a_e, b_e, torch.tensor([m])), alone.float(), f"expert {e} alone, depth pieces")
 
 
+@pytest.mark.parametrize("shrink", [8, 1])
+def test_config3_ragged_weight_gradient(ops, oracle, shrink):
+    # the weight gradient of the ragged configuration: Zipf depths from 0 to several thousand rows,
+    # at least four empty groups, tiles handed out by descending depth.  Shrunk against the CPU
+    # oracle; at full size against fp32 per expert on the GPU and CPU float64 blocks.
+    _announce("config3 weight gradient, shrink", shrink)
+    from grouped_gemm_amd import workloads
+    w = workloads.make(3, device="cuda", shrink=shrink)
+    sizes = w.batch_sizes
+    assert int((sizes == 0).sum()) >= 4
+    bg = ops.backend.gmm(w.a, w.grad, sizes.cuda(), trans_a=True)
+    assert torch.equal(bg, ops.backend.gmm(w.a, w.grad, sizes, trans_a=True))
+    if shrink > 1:
+        check(bg, oracle.gmm_loop(w.a.cpu(), w.grad.cpu(), sizes, trans_a=True), "weight gradient")
+    else:
+        starts = torch.cumsum(sizes, 0) - sizes
+        for e in range(len(sizes)):
+            s, m = int(starts[e]), int(sizes[e])
+            check(bg[e], w.a[s:s + m].float().t() @ w.grad[s:s + m].float(), f"expert {e}")
+        fp64_weight_gradient_check(w.a, w.grad, sizes, bg)
+    for e in (sizes == 0).nonzero().flatten().tolist():
+        assert (bg[e] == 0).all()
+
+
 def test_config4_weight_gradient_full_size(ops, oracle):
     _announce("config4 full")
     _full_size_case(ops, oracle, 4)
@@ -473,7 +497,18 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
     # tiles: two classes (all tiles but the runt rows, then the runt rows), each consecutive and
     # non-overlapping, together enough to cover each group's output
     first_class = got[:, 10] - got[:, 13]
-    assert np.array_equal(got[:, 9], np.cumsum(first_class) - first_class)
+    if trans_a:
+        # weight gradient: every group has the same number of tiles and they are handed out by
+        # descending depth, groups of equal depth in their own order (the reference's stable sort
+        # by k, csrc/grouped_gemm.cu:193-207): a permutation, depths non-increasing along it
+        position = np.empty(len(sizes), dtype=np.int64)
+        position[np.argsort(-np.array(sizes), kind="stable")] = np.arange(len(sizes))
+        assert np.array_equal(got[:, 9], position * first_class)
+        by_position = np.argsort(got[:, 9], kind="stable")
+        assert sorted(by_position.tolist()) == list(range(len(sizes)))
+        assert (np.diff(np.array(sizes)[by_position]) <= 0).all()
+    else:
+        assert np.array_equal(got[:, 9], np.cumsum(first_class) - first_class)
     assert np.array_equal(got[:, 12], first_class.sum() + np.cumsum(got[:, 13]) - got[:, 13])
     assert np.array_equal(got[:, 11], np.array(sizes))
     lib = ctypes.CDLL(os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so"))
@@ -835,10 +870,20 @@ def test_float16_autograd_and_mixed_dtypes(ops, oracle, trans_b):
 # ---- any hidden size, any alignment (the general kernels, and gmm's zero-padded copies instead)
 
 @pytest.fixture(params=[False, True], ids=["general-kernels", "padded-copies"])
-def odd_size_path(request, ops, monkeypatch):
-    """Both ways backend.gmm serves operands the streaming kernels do not take."""
-    monkeypatch.setattr(ops.backend, "PAD_ODD_SIZES", request.param)
-    return request.param
+def odd_size_path(request, ops):
+    """Both ways operands the streaming kernels do not take are served: the extension called
+    directly runs them copy-free on the general kernels, backend.gmm through zero-padded copies
+    on the streaming ones.  Returns gmm(a, b, batch_sizes, trans_a, trans_b, c=None)."""
+    if request.param:
+        return lambda a, b, bs, trans_a=False, trans_b=False, c=None: ops.backend.gmm(
+            a, b, bs, trans_a=trans_a, trans_b=trans_b, c=c)
+
+    def direct(a, b, bs, trans_a=False, trans_b=False, c=None):
+        if c is None:
+            c = ops.backend._allocate_output(a, b, bs, trans_a, trans_b)
+        ops.backend.backend.gmm(a, b, c, bs, trans_a, trans_b)
+        return c
+    return direct
 
 
 def _odd_cases(n, seed):
@@ -872,7 +917,7 @@ def test_hidden_sizes_that_are_not_multiples_of_8(ops, oracle, layout, dtype, od
         else:
             b = torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g).to(dtype)
         dev_bs = bs.cuda() if idx % 2 else bs
-        out = ops.backend.gmm(a.cuda(), b.cuda(), dev_bs, trans_a=trans_a, trans_b=trans_b)
+        out = odd_size_path(a.cuda(), b.cuda(), dev_bs, trans_a=trans_a, trans_b=trans_b)
         want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
         check(out, want, f"case {idx}: sizes={sizes} hin={hin} hout={hout}")
 
@@ -899,8 +944,41 @@ def test_operands_off_the_16_byte_boundary(ops, oracle, layout, odd_size_path):
     for by_a, by_b, by_c in [(1, 0, 0), (0, 2, 0), (0, 0, 4), (1, 3, 5)]:
         _announce("off boundary", layout, by_a, by_b, by_c)
         c = shifted(torch.zeros(want.shape, dtype=torch.bfloat16), by_c)
-        ops.backend.gmm(shifted(a, by_a), shifted(b, by_b), sizes.cuda(), trans_a=trans_a, trans_b=trans_b, c=c)
+        odd_size_path(shifted(a, by_a), shifted(b, by_b), sizes.cuda(), trans_a=trans_a, trans_b=trans_b, c=c)
         check(c, want, f"shifted by {by_a}, {by_b}, {by_c} elements")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_even_widths_with_b_stored_transposed_stream(ops, oracle, dtype):
+    # b stored transposed, depth a multiple of 8, width even but not a multiple of 8: rows of c
+    # start on 4-byte boundaries and the last 16-byte chunk of a row holds 2, 4 or 6 columns.  Runs
+    # on the streaming kernel as it is (no copies): exact row and column placement is checked with
+    # a sentinel around c, through the extension, through backend.gmm and with fused row indices.
+    for idx, (sizes, hin, hout) in enumerate([([300, 0, 17, 195], 264, 250), ([1, 255, 257, 64], 136, 262),
+                                              ([1000], 72, 518), ([5] * 40, 64, 6), ([33, 90], 6400, 1030),
+                                              ([40] * 30, 128, 772)]):
+        _announce("even width, NT", dtype, sizes, hin, hout)
+        g = torch.Generator().manual_seed(70 + idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        b = (torch.randn(len(sizes), hout, hin, generator=g) * hin ** -0.5).to(dtype)
+        want = oracle.gmm_loop(a, b, bs, trans_b=True)
+        # c in the middle of a larger buffer of sentinels, on a 4-byte boundary only
+        buf = torch.full(((t + 2) * hout + 2,), 7.0, dtype=dtype, device="cuda")
+        c = buf[hout + 2:hout + 2 + t * hout].view(t, hout)
+        assert c.data_ptr() % 4 == 0
+        ops.backend.backend.gmm(a.cuda(), b.cuda(), c, bs.cuda() if idx % 2 else bs, False, True)
+        check(c, want, f"case {idx}")
+        assert bool((buf[:hout + 2] == 7.0).all()) and bool((buf[hout + 2 + t * hout:] == 7.0).all())
+        out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda(), trans_b=True)
+        assert torch.equal(out, c)
+        perm = torch.randperm(t, generator=g).to(torch.int32).cuda()
+        c2 = torch.zeros(t, hout, dtype=dtype, device="cuda")
+        ops.backend.gmm_indexed(a.cuda(), b.cuda(), bs.cuda(), trans_b=True, c=c2, a_rows=perm, c_rows=perm)
+        want2 = torch.zeros_like(want)
+        want2[perm.long().cpu()] = oracle.gmm_loop(a[perm.long().cpu()], b, bs, trans_b=True)
+        check(c2, want2, f"case {idx}, gathered and scattered")
 
 
 def test_padded_copies_leave_tail_rows_alone(ops, oracle):
@@ -910,7 +988,6 @@ def test_padded_copies_leave_tail_rows_alone(ops, oracle):
     a = torch.randn(100, 33, generator=g).to(torch.bfloat16)
     b = torch.randn(3, 33, 50, generator=g).to(torch.bfloat16)
     c = torch.full((100, 50), 7.0, dtype=torch.bfloat16, device="cuda")
-    assert ops.backend.PAD_ODD_SIZES
     ops.backend.gmm(a.cuda(), b.cuda(), sizes.cuda(), c=c)
     check(c[:65], oracle.gmm_loop(a, b, sizes)[:65], "rows in use")
     assert bool((c[65:] == 7.0).all())
