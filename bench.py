@@ -28,13 +28,25 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2516.6   # 256 CU x 4096 flop/clk x 2.4 GHz, dense
 PEAK_HBM_GBPS = 8000.0
 
-# Bytes per launch between L2 and the fabric for the default workload, from two rocprofv3 --pmc
-# runs of this file (FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by a 1 GiB device copy, both in
-# KiB).  Profiled once, not in this run: `source` names the summary under profiles/ that holds the
-# figures, the commands and the revision of the kernel they were taken on.
-_TRAFFIC_SOURCE = ("profiles/gmm_kernel_mixtral_w1_hbm_traffic.md and profiles/gmm_kernel_configs_3_4_5_stats_and_traffic.md "
-                   "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the kernel revision with runt rows last and depth "
-                   "pieces; profiled once, not in this run)")
+# Bytes per launch between L2 and the fabric, from two rocprofv3 --pmc runs of this file per
+# configuration (FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by a 1 GiB device copy, both in KiB).
+# Profiled once, not in this run: the table belongs to one revision of the kernel sources, named by
+# the hash below (kernel_sources_sha16), and is reported only while the sources still have that
+# hash; the summary under profiles/ holds the figures, the commands and the commit.
+_TRAFFIC_KERNEL_SOURCES = ("gmm_kernel.hpp", "gmm_api.hip", "gmm_variants.hpp", "gmm_variants.def", "gmm_variant.hip")
+_TRAFFIC_KERNEL_SHA16 = "55c859b69b4a31bb"
+_TRAFFIC_SOURCE = ("profiles/gmm_kernel_hbm_traffic_configs_2_3_4_5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel "
+                   "sources sha16 " + _TRAFFIC_KERNEL_SHA16 + ", commit cfdacf2; profiled once, not in this run)")
+
+
+def kernel_sources_sha16():
+    """First 16 hex digits of the SHA-256 over the streaming kernel's sources."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in _TRAFFIC_KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "grouped_gemm_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def _traffic(fetch_kib, write_kib):
@@ -42,10 +54,10 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    2: {"fwd": _traffic(4088250, 917549), "agrad": _traffic(3325500, 290120), "bgrad": _traffic(2753350, 917545)},
-    3: {"fwd": _traffic(435980, 135184)},
-    4: {"bgrad": _traffic(2752720, 917516)},
-    5: {"fwd": _traffic(4359720, 262158), "agrad": _traffic(5455520, 917508), "bgrad": _traffic(1851630, 7342490)},
+    2: {"fwd": _traffic(4074410, 917538), "agrad": _traffic(3323260, 290088), "bgrad": _traffic(2753580, 917513)},
+    3: {"fwd": _traffic(447647, 135196)},
+    4: {"bgrad": _traffic(2752730, 917522)},
+    5: {"fwd": _traffic(4327950, 262153), "agrad": _traffic(5419070, 917507), "bgrad": _traffic(1851680, 7342530)},
 }
 
 
@@ -335,8 +347,15 @@ def main():
     value, roofline, slowest, kernel_ms = summarize(w, names, layout, ms_per_step, samples, args.accumulate)
     flops_gemm = w.flops_per_gemm()
     traffic = MEASURED_TRAFFIC.get(args.config, {}).get(slowest) if not (args.zeros or args.accumulate or args.flags or only) else None
-    roofline["traffic"] = round(traffic["bytes"]) if traffic else None
-    roofline["traffic_source"] = traffic["source"] if traffic else None
+    sources_now = kernel_sources_sha16()
+    if traffic and sources_now != _TRAFFIC_KERNEL_SHA16:
+        # the kernel sources have changed since the counters were read: no figure rather than a stale one
+        roofline["traffic"] = None
+        roofline["traffic_source"] = (f"not reported: the kernel sources (sha16 {sources_now}) are not the revision the "
+                                      f"counters were read on ({_TRAFFIC_KERNEL_SHA16})")
+    else:
+        roofline["traffic"] = round(traffic["bytes"]) if traffic else None
+        roofline["traffic_source"] = traffic["source"] if traffic else None
     metric, what = WORKLOAD_NAMES[args.config]
     if args.accumulate:
         metric, what = ("bf16 grouped-GEMM TFLOP/s, weight gradient accumulated into fp32",
@@ -357,7 +376,7 @@ def main():
         "data": "zeros (diagnostic, not a benchmark result)" if args.zeros else "synthetic",
         "config": {
             "workload": f"configs[{args.config - 1}]: {w.batch_sizes.numel()} experts, {w.tokens} routed rows, "
-                        f"{w.hidden_in}x{w.hidden_out}, {what}",
+                        f"{w.hidden_in}x{w.hidden_out}, " + (what if not only else "only: " + ", ".join(names)),
             "batch_sizes": w.batch_sizes.tolist() if w.batch_sizes.numel() <= 16 else "see workloads.make",
             "batch_sizes_on_device": True,
         },
