@@ -168,7 +168,8 @@ struct Route {
   int elem_bytes;
   bool indexed;        // any row index given
   bool indexed_fits;   // ... and a and c are within reach of the streaming kernels' 32-bit offsets
-  bool ragged_width;   // streaming kernel, b stored transposed, width even but not a multiple of 8
+  bool relaxed;        // streaming kernel on operands that are only 4-byte aligned (see classify)
+  bool ragged_width;   // ... with a width that is not a multiple of 8
   bool generic;        // the kernels of gmm_generic.hpp
   int vec;             // their vector width
   int64_t a_bytes, c_bytes;
@@ -195,14 +196,20 @@ Route classify(const gg_gmm_args& g) {
   const bool f8_streams = r.elem_bytes == 1 && (!swiglu || (trans_b && !r.indexed)) &&
                           (trans_a ? hidden_in % 16 == 0 && hidden_out % 16 == 0
                                    : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
-  // b stored transposed: rows of a and of b run along the depth, so only the depth has to be a
-  // multiple of 8; an even width that is not leaves rows of c on 4-byte boundaries, which the
-  // store epilogue of the streaming kernel handles (two-byte elements, c of the same type)
-  r.ragged_width = r.elem_bytes == 2 && trans_b && !trans_a && !swiglu && !g.accumulate_f32 &&
-                   hidden_in % 8 == 0 && hidden_out % 8 != 0 && hidden_out % 2 == 0 &&
-                   ((reinterpret_cast<uintptr_t>(g.a) | reinterpret_cast<uintptr_t>(g.b)) & 15) == 0 &&
-                   (reinterpret_cast<uintptr_t>(g.c) & 3) == 0;
-  r.generic = !r.ragged_width &&
+  // Two-byte elements with the plain store epilogue also stream from 4-byte boundaries: a 16-byte
+  // access needs no more than that, and the end of a buffer descriptor clips it dword by dword.
+  // What has to hold is that no 16-byte chunk mixes valid and foreign elements along the depth:
+  // rows that run along the depth (a, and b stored transposed) need a depth that is a multiple
+  // of 8.  Along the width a chunk may run past the row's end: what it picks up there lands in
+  // tile columns that are never stored.  So: hidden_in a multiple of 8 and hidden_out even, or,
+  // in the weight-gradient layout (both operands run along their widths), both even.  Rows of c
+  // then start on 4-byte boundaries and a row's last chunk may hold 2, 4 or 6 columns, which the
+  // store epilogue writes with narrower stores.
+  const bool aligned = hidden_in % 8 == 0 && hidden_out % 8 == 0 && (r.address_bits & 15) == 0;
+  r.relaxed = !aligned && r.elem_bytes == 2 && !swiglu && !g.accumulate_f32 && (r.address_bits & 3) == 0 &&
+              hidden_out % 2 == 0 && (trans_a ? hidden_in % 2 == 0 : hidden_in % 8 == 0);
+  r.ragged_width = r.relaxed && hidden_out % 8 != 0;
+  r.generic = !r.relaxed &&
               ((r.elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
                (r.address_bits & 15));
   r.generic = r.generic || (r.indexed && !r.indexed_fits);
@@ -445,6 +452,7 @@ uint64_t gg_workspace_bytes_for(const gg_gmm_args* args) {
   if (g.dtype < GG_DTYPE_BF16 || g.dtype > GG_DTYPE_F8E5M2 || g.hidden_in <= 0 || g.hidden_out <= 0) return 0;
   const Route r = classify(g);
   // (the kernels never cut tiles that are combined or scattered on their way out along the depth)
+  // (the fix-up of depth pieces stores 4 columns at a time: whole tiles and row pieces for ragged widths)
   if (r.generic || r.ragged_width || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
   if (g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ROW_PIECES)) return 0;
   if (!g.trans_a) {

@@ -1443,9 +1443,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
         constexpr int PITCH = Cfg::EPILOGUE_PITCH;
         const int in_row = lane & 31, in_half = lane >> 5;
         const int out_row = lane >> 3, out_chunk = lane & 7;
-        // NT layout: an even width that is not a multiple of 8 (rows of c then start on 4-byte
-        // boundaries only, and the last 16-byte chunk of a row holds 2, 4 or 6 columns)
-        const bool ragged_width = LAYOUT == kNT && uniform(ti.g.n & 7) != 0;
+        // an even width that is not a multiple of 8: rows of c then start on 4-byte boundaries
+        // only, and the last 16-byte chunk of a row holds 2, 4 or 6 columns
+        const bool ragged_width = uniform(ti.g.n & 7) != 0;
 #pragma unroll
         for (int i = 0; i < ML; ++i) {
           uint32_t row_off[4];
@@ -1466,7 +1466,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
               // (whole chunks only: for widths that are multiples of 8 the same as col < n)
               __builtin_amdgcn_raw_buffer_store_b128(v, rc, col + 8 <= ti.g.n ? at(row_off[r], col) : OOR, 0,
                                                      kStoreStreaming);
-              if constexpr (LAYOUT == kNT) {
+              {
                 if (ragged_width) {
                   const int valid = ti.g.n - col;   // columns of this lane's chunk that exist
                   const uint32_t off = at(row_off[r], col);

@@ -949,36 +949,57 @@ def test_operands_off_the_16_byte_boundary(ops, oracle, layout, odd_size_path):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_even_widths_with_b_stored_transposed_stream(ops, oracle, dtype):
-    # b stored transposed, depth a multiple of 8, width even but not a multiple of 8: rows of c
-    # start on 4-byte boundaries and the last 16-byte chunk of a row holds 2, 4 or 6 columns.  Runs
-    # on the streaming kernel as it is (no copies): exact row and column placement is checked with
-    # a sentinel around c, through the extension, through backend.gmm and with fused row indices.
-    for idx, (sizes, hin, hout) in enumerate([([300, 0, 17, 195], 264, 250), ([1, 255, 257, 64], 136, 262),
-                                              ([1000], 72, 518), ([5] * 40, 64, 6), ([33, 90], 6400, 1030),
-                                              ([40] * 30, 128, 772)]):
-        _announce("even width, NT", dtype, sizes, hin, hout)
+@pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
+def test_even_sizes_on_4_byte_boundaries_stream(ops, oracle, layout, dtype):
+    # Two-byte operands on 4-byte boundaries stream as they are (no copies) when no 16-byte chunk
+    # mixes elements along the depth: hidden_in a multiple of 8 and hidden_out even, or, with
+    # trans_a, both even.  Rows of c then start on 4-byte boundaries and the last 16-byte chunk of
+    # a row holds 2, 4 or 6 columns; chunks of b (and of a with trans_a) run past their rows' ends.
+    # Exact placement is checked with sentinels around c; a, b and c sit 4 bytes off the 16-byte
+    # boundary; through the extension, through backend.gmm and with fused row indices.
+    trans_a, trans_b = layout
+    cases = [([300, 0, 17, 195], 264, 250), ([1, 255, 257, 64], 136, 262), ([1000], 72, 518), ([5] * 40, 64, 6),
+             ([33, 90], 6400, 1030), ([40] * 30, 128, 772)]
+    if trans_a:
+        cases = [([300, 0, 17, 195], 262, 250), ([1, 255, 257, 64], 130, 266), ([1000], 70, 518), ([5] * 40, 6, 10),
+                 ([7000, 0, 6500], 258, 522), ([40] * 30, 772, 126)]
+
+    def off_boundary(x, fill=None):
+        # a view 4 bytes past a 16-byte boundary, with 2 sentinel elements in front and behind
+        buf = torch.full((x.numel() + 4,), 7.0 if fill is None else fill, dtype=x.dtype, device="cuda")
+        view = buf[2:2 + x.numel()].view(x.shape)
+        view.copy_(x)
+        assert view.data_ptr() % 16 == 4
+        return buf, view
+
+    for idx, (sizes, hin, hout) in enumerate(cases):
+        _announce("even sizes, 4-byte boundaries", layout, dtype, sizes, hin, hout)
         g = torch.Generator().manual_seed(70 + idx)
         bs = torch.tensor(sizes, dtype=torch.int64)
         t = int(bs.sum())
         a = torch.randn(t, hin, generator=g).to(dtype)
-        b = (torch.randn(len(sizes), hout, hin, generator=g) * hin ** -0.5).to(dtype)
-        want = oracle.gmm_loop(a, b, bs, trans_b=True)
-        # c in the middle of a larger buffer of sentinels, on a 4-byte boundary only
-        buf = torch.full(((t + 2) * hout + 2,), 7.0, dtype=dtype, device="cuda")
-        c = buf[hout + 2:hout + 2 + t * hout].view(t, hout)
-        assert c.data_ptr() % 4 == 0
-        ops.backend.backend.gmm(a.cuda(), b.cuda(), c, bs.cuda() if idx % 2 else bs, False, True)
-        check(c, want, f"case {idx}")
-        assert bool((buf[:hout + 2] == 7.0).all()) and bool((buf[hout + 2 + t * hout:] == 7.0).all())
-        out = ops.backend.gmm(a.cuda(), b.cuda(), bs.cuda(), trans_b=True)
+        if trans_a:
+            b = torch.randn(t, hout, generator=g).to(dtype)
+        else:
+            b = (torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g) * hin ** -0.5).to(dtype)
+        want = oracle.gmm_loop(a, b, bs, trans_a=trans_a, trans_b=trans_b)
+        _, da = off_boundary(a)
+        _, db = off_boundary(b)
+        cbuf, c = off_boundary(torch.zeros(want.shape, dtype=dtype))
+        cbuf.fill_(7.0)
+        ops.backend.backend.gmm(da, db, c, bs.cuda() if idx % 2 else bs, trans_a, trans_b)
+        scale = max(1.0, float(want.double().pow(2).mean().sqrt()))
+        check(c.float() / scale, want / scale, f"case {idx}")
+        assert bool((cbuf[:2] == 7.0).all()) and bool((cbuf[-2:] == 7.0).all())
+        out = ops.backend.gmm(da, db, bs.cuda(), trans_a=trans_a, trans_b=trans_b)
         assert torch.equal(out, c)
-        perm = torch.randperm(t, generator=g).to(torch.int32).cuda()
-        c2 = torch.zeros(t, hout, dtype=dtype, device="cuda")
-        ops.backend.gmm_indexed(a.cuda(), b.cuda(), bs.cuda(), trans_b=True, c=c2, a_rows=perm, c_rows=perm)
-        want2 = torch.zeros_like(want)
-        want2[perm.long().cpu()] = oracle.gmm_loop(a[perm.long().cpu()], b, bs, trans_b=True)
-        check(c2, want2, f"case {idx}, gathered and scattered")
+        if not trans_a:
+            perm = torch.randperm(t, generator=g).to(torch.int32).cuda()
+            c2 = torch.zeros(t, hout, dtype=dtype, device="cuda")
+            ops.backend.gmm_indexed(da, db, bs.cuda(), trans_b=trans_b, c=c2, a_rows=perm, c_rows=perm)
+            want2 = torch.zeros_like(want)
+            want2[perm.long().cpu()] = oracle.gmm_loop(a[perm.long().cpu()], b, bs, trans_b=trans_b)
+            check(c2, want2, f"case {idx}, gathered and scattered")
 
 
 def test_padded_copies_leave_tail_rows_alone(ops, oracle):
