@@ -455,9 +455,11 @@ uint64_t gg_workspace_bytes_for(const gg_gmm_args* args) {
   // (the fix-up of depth pieces stores 4 columns at a time: whole tiles and row pieces for ragged widths)
   if (r.generic || r.ragged_width || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
   if (g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ROW_PIECES)) return 0;
-  if (!g.trans_a) {
+  {
     const int64_t slice = r.elem_bytes == 1 ? 2 * gg::BK : gg::BK;   // depth elements per slice
-    if ((g.hidden_in + slice - 1) / slice < 2 * gg::kMinSlicesPerPiece) return 0;
+    // (weight-gradient layout: the depth is the group's row count, taken as the average)
+    const int64_t depth = g.trans_a ? g.tokens / (g.num_groups > 0 ? g.num_groups : 1) : g.hidden_in;
+    if ((depth + slice - 1) / slice < 2 * gg::kMinSlicesPerPiece) return 0;
   }
   return GG_WORKSPACE_BYTES;
 }

@@ -191,10 +191,8 @@ __global__ __launch_bounds__(THREADS) void gmm_generic_kernel(GenericParams gp, 
   __shared__ __attribute__((aligned(16))) char tile_b[BN * PITCH];
   build_schedule<LAYOUT, BM, BNS>(&sched, p, hs);
   __syncthreads();
-  if constexpr (LAYOUT == kTN) {
-    order_groups_by_depth(&sched, p.num_groups);
-    __syncthreads();
-  }
+  static_assert(sizeof(tile_a) >= kMaxGroups * sizeof(uint64_t), "the sort keys borrow a tile buffer");
+  if constexpr (LAYOUT == kTN) order_groups_by_depth(&sched, p.num_groups, reinterpret_cast<uint64_t*>(tile_a));
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;

@@ -217,7 +217,8 @@ int gg_gmm(const gg_gmm_args* args);
  * Bytes of workspace the call described by `args` can make use of: 0 when no launch of it ever
  * cuts tiles along the depth (general kernels, row indices, the SwiGLU epilogue, or a product too
  * shallow for depth pieces to pay: fewer than 96 depth slices of 64 two-byte or 128 one-byte
- * elements outside the trans_a layout), GG_WORKSPACE_BYTES otherwise.  Looks at the sizes, flags
+ * elements, the depth of the trans_a layout being the average rows per group),
+ * GG_WORKSPACE_BYTES otherwise.  Looks at the sizes, flags
  * and pointers' alignment only; args->workspace is ignored.  A caller that keeps workspaces
  * (one per stream) need not allocate one for calls this returns 0 for.  No counterpart in the
  * reference, which asks CUTLASS for its workspace size per call (csrc/grouped_gemm.cu:347-349).

@@ -423,8 +423,11 @@ def test_last_round_pieces_against_whole_tiles(ops, oracle, layout):
     # agree with each other far inside the tolerance, and each be the same bits on every call.
     trans_a, trans_b = layout
     whole_flag = ops.backend.backend.flag_whole_tiles
-    for idx, (sizes, hin, hout) in enumerate(_random_cases(16, seed=91 + int(trans_b) + 2 * int(trans_a))):
-        hin = hin * 8 if idx % 2 else hin     # deep enough for several depth pieces
+    cases = _random_cases(16, seed=91 + int(trans_b) + 2 * int(trans_a))
+    if trans_a:   # the depth is the groups' rows: deep groups, so that the cut runs along the depth
+        cases += [([13000, 0, 12500], 264, 520), ([6200, 6300], 136, 264), ([30000], 72, 200)]
+    for idx, (sizes, hin, hout) in enumerate(cases):
+        hin = hin * 8 if idx % 2 and idx < 16 else hin     # deep enough for several depth pieces
         _announce("pieces", layout, sizes, hin, hout)
         g = torch.Generator().manual_seed(idx)
         bs = torch.tensor(sizes, dtype=torch.int64)

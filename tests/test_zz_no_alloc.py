@@ -45,7 +45,7 @@ def test_no_alloc_entry_point_matches_workspace_entry_point(oracle, layout):
     # in use); the second call is smaller in every dimension; the third has no pieces at all
     calls = [([300, 40, 0, 129], 6400, 264), ([70, 0, 5], 6272, 136), ([64, 64], 128, 128)]
     if trans_a:
-        calls = [([7000, 0, 6500], 264, 520), ([6200, 3100], 136, 264), ([64, 64], 128, 128)]
+        calls = [([14000, 0, 13000], 264, 520), ([6300, 6200], 136, 264), ([64, 64], 128, 128)]
     for n, (sizes, hin, hout) in enumerate(calls):
         print("[case] no alloc", layout, sizes, hin, hout, flush=True)
         bs, t, a, b, shape = _case(100 + n, sizes, hin, hout, trans_a, trans_b)
