@@ -238,7 +238,8 @@ def other_paths(steps=7, warmup=4):
     workload (8 experts, 32768 rows, 4096 x 14336): fused row gather and scatter, the SwiGLU
     epilogue (the same b read as gate | up, so half the output width), float16, fp8 (e4m3, b as
     stored and b stored transposed, and the weight gradient), and hidden sizes that are not
-    multiples of 8 (through zero-padded copies, and on the general kernels)."""
+    multiples of 8 (odd ones through zero-padded copies and on the general kernels, even ones
+    as they are)."""
     import torch
     from grouped_gemm import backend
     from grouped_gemm_amd import workloads
@@ -282,18 +283,25 @@ def other_paths(steps=7, warmup=4):
     for key in ("float8_e4m3fn, b stored transposed", "float8_e4m3fn", "float8_e4m3fn, weight gradient (trans_a)"):
         res[key]["frac_of_fp8_mfma_peak"] = round(res[key]["TFLOP/s"] / (2 * PEAK_BF16_TFLOPS), 4)
     del a8, g8, wgrad
-    hin, hout = w.hidden_in - 4, w.hidden_out - 4
+    # odd hidden sizes: through zero-padded copies (what gmm does), and on the general kernels
+    hin, hout = w.hidden_in - 3, w.hidden_out - 3
     au, bu = w.a[:, :hin].contiguous(), w.b[:, :hin, :hout].contiguous()
     res[f"hidden sizes {hin} x {hout} (zero-padded copies, streaming kernel)"] = timed(
         lambda: backend.gmm(au, bu, sd), reps=2, f=2 * t * hin * hout)
     cu = torch.empty(t, hout, dtype=torch.bfloat16, device="cuda")
     res[f"hidden sizes {hin} x {hout} (general kernels, the extension called directly)"] = timed(
         lambda: backend.backend.gmm(au, bu, cu, sd, False, False), reps=2, f=2 * t * hin * hout)
-    del au, bu
-    # even sizes stream as they are: hidden_in a multiple of 8 and hidden_out even
-    bn = w.b[:, :, :hout].contiguous()
-    res[f"hidden sizes {w.hidden_in} x {hout} (streaming kernel, no copies)"] = timed(
-        lambda: backend.gmm(w.a, bn, sd, c=cu), f=2 * t * w.hidden_in * hout)
+    del au, bu, cu
+    # even hidden sizes that are no multiples of 8 stream as they are: the forward product and the
+    # input gradient (whose rows run along the ragged hidden size) of such a layer
+    hin, hout = w.hidden_in - 4, w.hidden_out - 4
+    au, bu = w.a[:, :hin].contiguous(), w.b[:, :hin, :hout].contiguous()
+    cu = torch.empty(t, hout, dtype=torch.bfloat16, device="cuda")
+    res[f"hidden sizes {hin} x {hout} (streaming kernel, no copies)"] = timed(
+        lambda: backend.gmm(au, bu, sd, c=cu), f=2 * t * hin * hout)
+    gu = torch.empty(t, hin, dtype=torch.bfloat16, device="cuda")
+    res[f"hidden sizes {hin} x {hout}, input gradient (streaming kernel, no copies)"] = timed(
+        lambda: backend.gmm(cu, bu, sd, trans_b=True, c=gu), f=2 * t * hin * hout)
     return res
 
 

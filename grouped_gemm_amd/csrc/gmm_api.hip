@@ -170,6 +170,7 @@ struct Route {
   bool indexed_fits;   // ... and a and c are within reach of the streaming kernels' 32-bit offsets
   bool relaxed;        // streaming kernel on operands that are only 4-byte aligned (see classify)
   bool ragged_width;   // ... with a width that is not a multiple of 8
+  bool ragged_depth;   // ... with rows along a depth that is not a multiple of 8
   bool generic;        // the kernels of gmm_generic.hpp
   int vec;             // their vector width
   int64_t a_bytes, c_bytes;
@@ -198,17 +199,20 @@ Route classify(const gg_gmm_args& g) {
                                    : hidden_in % 16 == 0 && (trans_b || hidden_out % 16 == 0));
   // Two-byte elements with the plain store epilogue also stream from 4-byte boundaries: a 16-byte
   // access needs no more than that, and the end of a buffer descriptor clips it dword by dword.
-  // What has to hold is that no 16-byte chunk mixes valid and foreign elements along the depth:
-  // rows that run along the depth (a, and b stored transposed) need a depth that is a multiple
-  // of 8.  Along the width a chunk may run past the row's end: what it picks up there lands in
-  // tile columns that are never stored.  So: hidden_in a multiple of 8 and hidden_out even, or,
-  // in the weight-gradient layout (both operands run along their widths), both even.  Rows of c
-  // then start on 4-byte boundaries and a row's last chunk may hold 2, 4 or 6 columns, which the
-  // store epilogue writes with narrower stores.
+  // Both hidden sizes have to be even (rows then start on 4-byte boundaries).  Along the width a
+  // chunk may run past the row's end: what it picks up there lands in tile columns that are never
+  // stored, and a row of c whose last chunk holds 2, 4 or 6 columns is finished with narrower
+  // stores.  Along the depth (rows of a, and of b stored transposed; not in the weight-gradient
+  // layout, where both operands run along their widths) such a chunk would add the next row's
+  // first values to the sums: a kernel variant clears them in LDS before the slice is multiplied
+  // (WideRaggedDepth; plain rows only, no row indices).
   const bool aligned = hidden_in % 8 == 0 && hidden_out % 8 == 0 && (r.address_bits & 15) == 0;
   r.relaxed = !aligned && r.elem_bytes == 2 && !swiglu && !g.accumulate_f32 && (r.address_bits & 3) == 0 &&
-              hidden_out % 2 == 0 && (trans_a ? hidden_in % 2 == 0 : hidden_in % 8 == 0);
+              hidden_out % 2 == 0 && hidden_in % 2 == 0;
   r.ragged_width = r.relaxed && hidden_out % 8 != 0;
+  r.ragged_depth = !trans_a && hidden_in % 8 != 0;
+  if (r.ragged_depth && r.indexed) r.relaxed = false;
+  r.ragged_depth = r.ragged_depth && r.relaxed;
   r.generic = !r.relaxed &&
               ((r.elem_bytes != 2 && !f8_streams) || hidden_in % 8 != 0 || hidden_out % 8 != 0 ||
                (r.address_bits & 15));
@@ -297,14 +301,15 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   // its time than reading, adding and writing; shallow groups: bound by the traffic of c, the reverse
   const int variant_epilogue = out_f32 && tokens >= (int64_t)kShallowBelow * num_groups ? gg::kEpiAccF32Atomic : epilogue;
   // (the short tile shape exists for two-byte elements, the plain epilogue and rows in place only)
-  const bool short_shape = !generic && !swiglu && !indexed && elem_bytes == 2 &&
+  const bool short_shape = !generic && !swiglu && !indexed && elem_bytes == 2 && !route.ragged_depth &&
                            use_short_shape(num_groups, tokens, trans_a);
   const int bm = generic ? gg::kGenericTileM : (short_shape ? Short::BM : Wide::BM);
   // output columns per tile: half the tile's width when it holds gate and up columns
   const int bn = (generic ? gg::kGenericTileN : (short_shape ? Short::BN : Wide::BN)) / (swiglu ? 2 : 1);
   const gg::VariantOps* variant = nullptr;
   if (!generic) {
-    variant = find_variant(g.dtype, layout, short_shape ? Short::kId : Wide::kId, variant_epilogue, indexed ? 1 : 0);
+    const int shape = route.ragged_depth ? gg::WideRaggedDepth::kId : (short_shape ? Short::kId : Wide::kId);
+    variant = find_variant(g.dtype, layout, shape, variant_epilogue, indexed ? 1 : 0);
     if (variant == nullptr) return fail(GG_EINVAL, "no kernel for this combination of arguments");
   }
 
@@ -330,6 +335,10 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
   static_assert(GG_FLAG_WHOLE_TILES == gg::kFlagWholeTiles && GG_FLAG_ONE_CLASS == gg::kFlagOneClass &&
                 GG_FLAG_ROW_PIECES == gg::kFlagRowPieces, "the header's flags are the kernel's");
   p.flags = g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ONE_CLASS | GG_FLAG_ROW_PIECES);
+  // (ragged widths: the fix-up of depth pieces stores 4 columns at a time; ragged depths: the
+  // kernel looks for the ragged chunks in the slice hidden_in / 64 of tiles that start at depth 0.
+  // Whole tiles and row pieces only, for both.)
+  const bool no_depth_pieces = route.ragged_width || route.ragged_depth;
   p.sched_out = nullptr;
   if (static_scratch) {
     if (g.workspace != nullptr)
@@ -341,14 +350,13 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     p.ws_slots = (int32_t)(((uint64_t)GG_WORKSPACE_BYTES - gg::kWsCounterBytes) /
                            ((uint64_t)bm * bn * (swiglu ? 2 : 1) * 4));
     if (p.ws_slots > 1024) p.ws_slots = 1024;
-    // (the fix-up of depth pieces stores 4 columns at a time: whole tiles and row pieces only)
-    if (route.ragged_width) p.ws_slots = 0;
+    if (no_depth_pieces) p.ws_slots = 0;
     // Every call on this device shares the array and finds what the last call left: the arrival
     // counters must start at zero (a fill kernel, not a memset: callers may be capturing a graph).
     hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(gg::kWsCounterBytes / 4), 0, stream,
                        reinterpret_cast<int*>(info.scratch));
     GG_HIP(hipGetLastError());
-  } else if (g.workspace != nullptr && !generic && !route.ragged_width) {
+  } else if (g.workspace != nullptr && !generic && !no_depth_pieces) {
     if (reinterpret_cast<uintptr_t>(g.workspace) & 255)
       return fail(GG_ELIMIT, "the workspace must be 256-byte aligned");
     const uint64_t slot_bytes = (uint64_t)bm * bn * (swiglu ? 2 : 1) * 4;
@@ -453,7 +461,7 @@ uint64_t gg_workspace_bytes_for(const gg_gmm_args* args) {
   const Route r = classify(g);
   // (the kernels never cut tiles that are combined or scattered on their way out along the depth)
   // (the fix-up of depth pieces stores 4 columns at a time: whole tiles and row pieces for ragged widths)
-  if (r.generic || r.ragged_width || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
+  if (r.generic || r.ragged_width || r.ragged_depth || r.indexed || g.epilogue == GG_EPILOGUE_SWIGLU) return 0;
   if (g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ROW_PIECES)) return 0;
   {
     const int64_t slice = r.elem_bytes == 1 ? 2 * gg::BK : gg::BK;   // depth elements per slice

@@ -670,6 +670,21 @@ struct DepthMajor {
     }
     load_to_lds_16(sl.rsrc, v, uniform(lds_address(dst) + (I * NT + wave * 64) * 16));
   }
+
+  // A depth that is even but no multiple of 8: the 16-byte chunk that holds a row's last depth
+  // values also holds the first values of the next row in memory (only behind the last row does the
+  // descriptor end).  Once the slice with that chunk has landed, every thread clears the foreign
+  // dwords of its rows' chunks in the LDS tile at `tile`, so that nothing of another row, not even
+  // a NaN against a zero, reaches a sum.  tail = depth values of the slice that exist.
+  __device__ static __forceinline__ void clear_depth_tail(char* tile, int tail) {
+    const int chunk = tail >> 3, first_dword = (tail & 7) >> 1;
+    for (int row = threadIdx.x; row < R; row += NT) {
+      uint32_t* at = reinterpret_cast<uint32_t*>(tile + row * (BK * 2) + ((chunk ^ ((row / RP) % CPR)) << 4));
+#pragma unroll
+      for (int d = 1; d < 4; ++d)
+        if (d >= first_dword) at[d] = 0u;
+    }
+  }
 };
 
 // F8 (one-byte elements, seen two to one as W two-byte elements per depth row): 32-byte segment
@@ -1026,8 +1041,9 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
 // (gradient accumulation, weight-gradient layout); or, with gate | up columns in b, combined to
 // silu(gate) * up and stored half as wide.
 // INDEXED: rows of a are fetched and rows of c stored through p.a_rows / p.c_rows (NN and NT).
+// RAGGED_DEPTH: hidden_in is even but no multiple of 8 (NN and NT, two-byte elements, plain store).
 template <int DT, int LAYOUT, int BM, int BN, int BK, int STAGES, int WAVES_M, int WAVES_N,
-          int EPI = kEpiStore, bool INDEXED = false>
+          int EPI = kEpiStore, bool INDEXED = false, bool RAGGED_DEPTH = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p, HostSizes hs) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   using Cfg = GmmConfig<LAYOUT, BM, BN, BK, STAGES, WAVES_M, WAVES_N>;
@@ -1075,7 +1091,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
 
   // (a tile that is combined or scattered on its way out is never cut along the depth: the
   // fix-up of the depth pieces stores plain tiles)
-  constexpr bool DEPTH_PIECES = !(GATE_UP || INDEXED);
+  constexpr bool DEPTH_PIECES = !(GATE_UP || INDEXED || RAGGED_DEPTH);
   TailPlan plan = plan_tail<LAYOUT, DEPTH_PIECES>(
       uniform(sched->tile_start[p.num_groups]) + uniform(sched->runt_start[p.num_groups]),
       (int)gridDim.x, p, BK_ELEMS);
@@ -1214,8 +1230,25 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     return unpack_tile(words);
   };
   TileInfo ti = next_tile();
+  // RAGGED_DEPTH: hidden_in is even but no multiple of 8.  No depth pieces then (every tile starts at
+  // depth 0), so the ragged chunks are in slice hidden_in / BK of every tile.  Once a buffer holds
+  // that slice, complete for every wave, what its ragged chunks picked up from the rows behind is
+  // cleared before any wave reads a fragment from it.
+  static_assert(!RAGGED_DEPTH || (LAYOUT != kTN && !F8 && !GATE_UP && !INDEXED), "");
+  const int tail_slice = RAGGED_DEPTH ? p.hidden_in / BK : -1;
+  auto clear_tail = [&](int buf) {
+    if constexpr (RAGGED_DEPTH) {
+      char* st = smem + uniform(buf) * Cfg::STAGE_BYTES;
+      const int tail = p.hidden_in % BK;
+      if constexpr (Cfg::A_DEPTH_MAJOR) ALoad::clear_depth_tail(st, tail);
+      if constexpr (Cfg::B_DEPTH_MAJOR) BLoad::clear_depth_tail(st + Cfg::A_BYTES, tail);
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      block_barrier();
+    }
+  };
   wait_vmcnt<3 * QUARTER_LOADS>();   // the first slice is in
   block_barrier();
+  if (RAGGED_DEPTH && tail_slice == 0) clear_tail(0);
   static_for<2 * UNITS>([&](auto u) {
     constexpr int uu = decltype(u)::value;
     read_unit(std::integral_constant<int, uu % UNITS>{}, std::integral_constant<int, uu / UNITS>{}, IMB{}, 0);
@@ -1307,6 +1340,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       // the next slice has landed for every wave (only this slice's two quarters may be pending)
       wait_vmcnt<2 * QUARTER_LOADS>();
       block_barrier();
+      if (RAGGED_DEPTH && uniform(kt + 1 == ti.nk ? 0 : kt + 1) == tail_slice) clear_tail(y);
       step(I3{}, I2{}, IMB{}, I0{}, IQ2{}, IQ{}, y, x);
       x = uniform(y);
     }

@@ -28,7 +28,8 @@ using Cfg = GmmConfig<V::LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_
 
 const void* kernel_address() {
   return reinterpret_cast<const void*>(
-      &gmm_kernel<V::DT, V::LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, V::EPI, V::INDEXED>);
+      &gmm_kernel<V::DT, V::LAYOUT, S::BM, S::BN, BK, STAGES, S::WAVES_M, S::WAVES_N, V::EPI, V::INDEXED,
+                  S::RAGGED_DEPTH>);
 }
 
 hipError_t prepare() {

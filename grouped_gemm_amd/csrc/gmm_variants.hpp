@@ -17,9 +17,18 @@ constexpr int BK = 64, STAGES = 2;
 // wide shape: its ragged dimension is the depth, not the rows.
 struct Wide {
   static constexpr int kId = 0, BM = 256, BN = 256, WAVES_M = 2, WAVES_N = 2;
+  static constexpr bool RAGGED_DEPTH = false;
 };
 struct Short {
   static constexpr int kId = 1, BM = 128, BN = 256, WAVES_M = 1, WAVES_N = 4;
+  static constexpr bool RAGGED_DEPTH = false;
+};
+// The wide shape for a hidden_in that is even but no multiple of 8, in the layouts whose rows run
+// along the depth: the kernel then clears, in LDS, what the last 16-byte chunk of a row picks up
+// from the next row (DepthMajor::clear_depth_tail), and cuts no tile along the depth.
+struct WideRaggedDepth : Wide {
+  static constexpr int kId = 2;
+  static constexpr bool RAGGED_DEPTH = true;
 };
 
 struct VariantOps {

@@ -99,8 +99,8 @@ int gg_init(void);
  * Limits (GG_ELIMIT): hidden_in and hidden_out below 2^22; tokens below 2^31.  Hidden sizes that
  * are multiples of 8 with a, b and c on 16-byte boundaries (the alignment the reference's kernel
  * configuration assumes, csrc/grouped_gemm.cu:41-66) run on the streaming kernels, and so do
- * operands on 4-byte boundaries with an even hidden_out and a hidden_in that is a multiple of 8
- * (with trans_a: even); other sizes and alignments run on slower, general kernels (see gg_gmm).
+ * operands on 4-byte boundaries with even hidden sizes; other sizes and alignments run on slower,
+ * general kernels (see gg_gmm).
  */
 int gg_gmm_bf16(const void* a, const void* b, void* c, const int64_t* batch_sizes,
                 int batch_sizes_on_device, int64_t num_groups, int64_t tokens,
@@ -137,9 +137,8 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  *                 8, :469).  Multiples of 8 with 16-byte aligned two-byte operands run on the
  *                 streaming kernels, and so do fp8 operands whose contiguous dimensions are
  *                 multiples of 16, and, with the plain epilogue (no SwiGLU, no fp32 accumulation),
- *                 two-byte operands on 4-byte boundaries with an even hidden_out and a hidden_in
- *                 that is a multiple of 8 (with trans_a: even); everything else on slower,
- *                 general ones.
+ *                 two-byte operands on 4-byte boundaries with even hidden sizes; everything else
+ *                 (odd sizes, 2-byte boundaries) on slower, general ones.
  *   a_row_index   int32[tokens] on the device, or NULL: row r of the product's left operand is
  *                 row a_row_index[r] of `a` (a gather fused into the load: `a` is the tensor
  *                 before the permutation that sorts rows by group, and may have any number of

@@ -954,9 +954,9 @@ def test_operands_off_the_16_byte_boundary(ops, oracle, layout, odd_size_path):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("layout", [(False, False), (False, True), (True, False)])
 def test_even_sizes_on_4_byte_boundaries_stream(ops, oracle, layout, dtype):
-    # Two-byte operands on 4-byte boundaries stream as they are (no copies) when no 16-byte chunk
-    # mixes elements along the depth: hidden_in a multiple of 8 and hidden_out even, or, with
-    # trans_a, both even.  Rows of c then start on 4-byte boundaries and the last 16-byte chunk of
+    # Two-byte operands on 4-byte boundaries stream as they are (no copies) when both hidden sizes
+    # are even; here no 16-byte chunk mixes elements along the depth (hidden_in a multiple of 8, or
+    # trans_a; the other depths have the test below).  Rows of c start on 4-byte boundaries and the last 16-byte chunk of
     # a row holds 2, 4 or 6 columns; chunks of b (and of a with trans_a) run past their rows' ends.
     # Exact placement is checked with sentinels around c; a, b and c sit 4 bytes off the 16-byte
     # boundary; through the extension, through backend.gmm and with fused row indices.
@@ -1003,6 +1003,61 @@ def test_even_sizes_on_4_byte_boundaries_stream(ops, oracle, layout, dtype):
             want2 = torch.zeros_like(want)
             want2[perm.long().cpu()] = oracle.gmm_loop(a[perm.long().cpu()], b, bs, trans_b=trans_b)
             check(c2, want2, f"case {idx}, gathered and scattered")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_even_depths_that_are_no_multiple_of_8_stream(ops, oracle, trans_b, dtype):
+    # hidden_in even but no multiple of 8, in the layouts whose rows run along the depth: the
+    # 16-byte chunk with a row's last 2, 4 or 6 depth values also holds the first values of the next
+    # row in memory, which the kernel clears in LDS.  Those first values are poisoned here: one row
+    # of a (and, stored transposed, one row of b per group) starts with NaNs, so its own outputs are
+    # NaN and every other output must be finite and right.  Depths below one slice, ragged in the
+    # first, a middle and the last chunk of a slice, and deep enough for depth pieces otherwise.
+    cases = [([300, 0, 17, 195], 262, 250), ([1, 255, 257, 64], 130, 264), ([1000], 70, 518), ([5] * 40, 6, 16),
+             ([33, 90], 6404, 1032), ([40] * 30, 66, 772), ([70, 300], 1022, 130), ([129], 58, 72)]
+    for idx, (sizes, hin, hout) in enumerate(cases):
+        _announce("even depth, no multiple of 8", trans_b, dtype, sizes, hin, hout)
+        g = torch.Generator().manual_seed(90 + idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(dtype)
+        b = (torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g) * hin ** -0.5).to(dtype)
+        bad_row = t // 2
+        a[bad_row, :min(6, hin)] = float("nan")
+        bad_col = hout // 3
+        if trans_b:
+            b[:, bad_col, :min(6, hin)] = float("nan")
+        want = oracle.gmm_loop(a, b, bs, trans_b=trans_b)
+        finite = torch.ones_like(want, dtype=torch.bool)
+        finite[bad_row] = False
+        if trans_b:
+            finite[:, bad_col] = False
+        assert bool(torch.isnan(want[~finite]).all()) and bool(torch.isfinite(want[finite]).all())
+        da, db = a.cuda(), b.cuda()
+        c = torch.full((t + 1, hout), 7.0, dtype=dtype, device="cuda")
+        ops.backend.backend.gmm(da, db, c[:t], bs.cuda() if idx % 2 else bs, False, trans_b)
+        got = c[:t].cpu()
+        assert bool(torch.isnan(got[~finite]).all()), f"case {idx}: poisoned outputs"
+        assert bool(torch.isfinite(got[finite]).all()), f"case {idx}: a NaN of a neighbouring row reached a sum"
+        clean = lambda x: torch.where(finite, x.float(), torch.zeros((), dtype=torch.float32))
+        check(clean(got), clean(want), f"case {idx}")
+        assert bool((c[t] == 7.0).all())
+        out = ops.backend.gmm(da, db, bs.cuda(), trans_b=trans_b)
+        assert torch.equal(clean(out.cpu()), clean(got))
+        # rows through indices, and the workspace the binding would fetch: none for these sizes
+        perm = torch.randperm(t, generator=g).to(torch.int32).cuda()
+        c2 = torch.zeros(t, hout, dtype=dtype, device="cuda")
+        ops.backend.gmm_indexed(da, db, bs.cuda(), trans_b=trans_b, c=c2, a_rows=perm, c_rows=perm)
+        rows = perm.long().cpu()
+        want2 = torch.zeros_like(want)
+        want2[rows] = oracle.gmm_loop(a[rows], b, bs, trans_b=trans_b)
+        finite2 = torch.isfinite(want2)
+        got2 = c2.cpu()
+        assert bool((torch.isfinite(got2) == finite2).all()), f"case {idx}, gathered and scattered: NaN placement"
+        zero = torch.zeros((), dtype=torch.float32)
+        check(torch.where(finite2, got2.float(), zero), torch.where(finite2, want2.float(), zero),
+              f"case {idx}, gathered and scattered")
 
 
 def test_padded_copies_leave_tail_rows_alone(ops, oracle):
