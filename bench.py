@@ -137,9 +137,19 @@ WORKLOAD_NAMES = {
 }
 
 
-def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0, only=None):
+# After an idle period the device runs through a power-management transient: about 5 launches at a
+# boosted clock, then up to 35 % slower than the steady state, which it reaches again after 20-25
+# ms of continuous work.  A workload whose step takes a fraction of a millisecond would be timed
+# inside that transient after a handful of warm-up steps, so warm-up goes on until the device has
+# been busy this long (the default workload's 10 warm-up steps are 88 ms: nothing is added there).
+WARMUP_BUSY_MS = 60.0
+
+
+def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0, only=None, min_timed_ms=0.0):
     """Times the grouped GEMMs of one configuration; returns (workload, names, layout, ms_per_step,
-    per-launch samples in ms)."""
+    per-launch samples in ms, steps timed, warm-up steps run).  At least `warmup` warm-up steps,
+    more until the device has been busy for WARMUP_BUSY_MS; at least `steps` timed steps, more
+    until they cover `min_timed_ms`."""
     import torch
     from grouped_gemm import backend
     from grouped_gemm_amd import workloads
@@ -182,9 +192,25 @@ def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0, 
             else:
                 calls[n]()
 
-    for _ in range(warmup):
+    # (the first step also loads the kernels: the step time is taken from the steps after it)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    for i in range(warmup):
         step()
+        if i == 0:
+            marks[0].record()
+    if warmup < 2:
+        step()
+        warmup += 1
+    marks[1].record()
     torch.cuda.synchronize()
+    step_ms = max(marks[0].elapsed_time(marks[1]) / (warmup - 1), 1e-3)
+    if step_ms * warmup < WARMUP_BUSY_MS:
+        extra = min(int((WARMUP_BUSY_MS - step_ms * warmup) / step_ms) + 1, 2000)
+        for _ in range(extra):
+            step()
+        torch.cuda.synchronize()
+        warmup += extra
+    steps = max(steps, min(int(min_timed_ms / step_ms) + 1, 500))
     events = {n: [] for n in names}
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -192,7 +218,7 @@ def run_workload(config, steps, warmup, accumulate=False, zeros=False, flags=0, 
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) / steps * 1e3
     samples = {n: sorted(a.elapsed_time(b) for a, b in ev) for n, ev in events.items()}
-    return w, names, layout, ms_per_step, samples
+    return w, names, layout, ms_per_step, samples, steps, warmup
 
 
 def summarize(w, names, layout, ms_per_step, samples, accumulate=False):
@@ -351,8 +377,8 @@ def main():
         print(json.dumps({"copied_bytes": args.copy_bytes, "times": 5}))
         return
     only = tuple(args.only.split(",")) if args.only else None
-    w, names, layout, ms_per_step, samples = run_workload(args.config, args.steps, args.warmup,
-                                                          args.accumulate, args.zeros, args.flags, only)
+    w, names, layout, ms_per_step, samples, _, warmup_run = run_workload(args.config, args.steps, args.warmup,
+                                                                         args.accumulate, args.zeros, args.flags, only)
     value, roofline, slowest, kernel_ms = summarize(w, names, layout, ms_per_step, samples, args.accumulate)
     flops_gemm = w.flops_per_gemm()
     traffic = MEASURED_TRAFFIC.get(args.config, {}).get(slowest) if not (args.zeros or args.accumulate or args.flags or only) else None
@@ -376,7 +402,7 @@ def main():
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
-        "warmup": args.warmup,
+        "warmup": warmup_run,   # args.warmup, or more for a short step (see WARMUP_BUSY_MS)
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -448,13 +474,14 @@ def main():
         for cfg, acc, only in ((3, False, None), (3, False, ("bgrad",)), (4, False, None), (4, True, None),
                                (5, False, None)):
             torch.cuda.empty_cache()
-            res = run_workload(cfg, min(args.steps, 10), min(args.warmup, 3), accumulate=acc, only=only)
-            v, roof, _, _ = summarize(*res, accumulate=acc)
+            res = run_workload(cfg, min(args.steps, 10), min(args.warmup, 3), accumulate=acc, only=only,
+                               min_timed_ms=30.0)
+            v, roof, _, _ = summarize(*res[:5], accumulate=acc)
             others[f"configs[{cfg - 1}]" + (" accumulate" if acc else "") + (" weight gradient" if only else "")] = {
                 "workload": ("weight-gradient grouped GEMM of the same workload" if only else
                              WORKLOAD_NAMES[cfg][1] if not acc else "weight gradient added to an fp32 output"),
                 "experts": res[0].batch_sizes.numel(), "rows": res[0].tokens,
-                "hidden": f"{res[0].hidden_in}x{res[0].hidden_out}", "steps": min(args.steps, 10),
+                "hidden": f"{res[0].hidden_in}x{res[0].hidden_out}", "steps": res[5], "warmup": res[6],
                 "ms_per_step": round(res[3], 4), "TFLOP/s": round(v, 2),
                 "bound": roof["bound"], "achieved": roof["achieved"], "unit": roof["unit"], "frac": roof["frac"],
                 "slowest_kernel": roof["kernel"],
