@@ -94,6 +94,8 @@ enum : int {   // debugging switches, for comparing the ways a call can be sched
   kFlagWholeTiles = 1,    // never cut the tiles of the last round into pieces
   kFlagOneClass = 2,      // hand out runt rows in place, not after all other tiles
   kFlagRowPieces = 4,     // ignore the workspace: cut along the rows only
+  kFlagGroupOrder = 8,    // NN and NT layouts: never hand out the groups' tiles by tile height
+  kFlagByHeight = 16,     // set by the host side (never by callers): hand them out by tile height
 };
 
 // Workspace layout: kWsCounterBytes of int32 arrival counters (one per tile of the last round; all
@@ -167,11 +169,13 @@ struct Sched {
   int32_t tile_start[kMaxGroups + 1];  // exclusive prefix sum of the first class's tiles
   int32_t runt_start[kMaxGroups + 1];  // exclusive prefix sum of the runt rows' tiles
   int32_t arrived;                     // broadcast slot for the arrival count of a depth piece
-  // Weight-gradient layout only: the groups by descending depth (order[q] is the group whose tiles
-  // are handed out q-th).  Every group has the same number of tiles there and a tile's cost is its
-  // group's depth, so the deepest groups go first and the shallow ones fill the end of the launch:
-  // what the reference's sort by k does for its scheduler (csrc/grouped_gemm.cu:193-207,
-  // csrc/fill_arguments.cuh:80-81).  Results do not depend on it.
+  // order[q] is the group whose tiles are handed out q-th.  Weight-gradient layout: by descending
+  // depth.  Every group has the same number of tiles there and a tile's cost is its group's depth,
+  // so the deepest groups go first and the shallow ones fill the end of the launch: what the
+  // reference's sort by k does for its scheduler (csrc/grouped_gemm.cu:193-207,
+  // csrc/fill_arguments.cuh:80-81).  Other layouts, with kFlagByHeight: by descending tile height
+  // (tile_start and runt_start then count in that order); without: not used.  Results do not
+  // depend on it.
   int16_t order[kMaxGroups];
 };
 
@@ -419,19 +423,23 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
   }
 }
 
-// Run by every thread of the workgroup after build_schedule and a barrier (weight-gradient layout
-// only); ends with a barrier.  A bitonic sort in LDS of one 64-bit key per group, depth above
-// and 0xffff - index below, so that groups of equal depth keep their order (what the reference's
-// stable sort gives); `keys` is scratch for kMaxGroups keys (the tile buffers are not in use yet).
-__device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, uint64_t* keys) {
+// Run by every thread of the workgroup after build_schedule and a barrier; ends with a barrier.
+// Fills Sched::order with the groups by descending key_of(group), groups of equal key in their
+// own order (what the reference's stable sort gives); `keys` is scratch for kMaxGroups 64-bit
+// words (the tile buffers are not in use yet).
+template <typename KeyFn>
+__device__ __forceinline__ void order_groups(Sched* s, int num_groups, uint64_t* keys, KeyFn key_of) {
   // Up to a few hundred groups it is quicker to count, per group, the groups that go before it
-  // (no barriers; measured equal at 256 groups, 12 us slower than the sort at 512).
+  // (measured equal at 256 groups, 12 us slower than the sort at 512).
   if (num_groups <= 256) {
+    uint32_t* key32 = reinterpret_cast<uint32_t*>(keys);
+    for (int e = threadIdx.x; e < num_groups; e += blockDim.x) key32[e] = (uint32_t)key_of(e);
+    __syncthreads();
     for (int e = threadIdx.x; e < num_groups; e += blockDim.x) {
-      const int mine = s->rows[e];
+      const uint32_t mine = key32[e];
       int before = 0;
       for (int j = 0; j < num_groups; ++j) {
-        const int other = s->rows[j];   // (the same address in every lane: a broadcast read)
+        const uint32_t other = key32[j];   // (the same address in every lane: a broadcast read)
         before += (other > mine || (other == mine && j < e)) ? 1 : 0;
       }
       s->order[before] = (int16_t)e;
@@ -439,10 +447,11 @@ __device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, 
     __syncthreads();
     return;
   }
+  // A bitonic sort in LDS of one 64-bit word per group, key above and 0xffff - index below.
   int n = 2;
   while (n < num_groups) n <<= 1;
   for (int i = threadIdx.x; i < n; i += blockDim.x)
-    keys[i] = i < num_groups ? ((uint64_t)(uint32_t)s->rows[i] << 16) | (uint64_t)(0xffff - i) : 0;   // padding sorts last
+    keys[i] = i < num_groups ? ((uint64_t)(uint32_t)key_of(i) << 16) | (uint64_t)(0xffff - i) : 0;   // padding sorts last
   __syncthreads();
   for (int k = 2; k <= n; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
@@ -461,6 +470,60 @@ __device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, 
     }
   }
   for (int i = threadIdx.x; i < num_groups; i += blockDim.x) s->order[i] = (int16_t)(0xffff - (int)(keys[i] & 0xffff));
+  __syncthreads();
+}
+
+// Weight-gradient layout: the groups by descending depth.
+__device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, uint64_t* keys) {
+  order_groups(s, num_groups, keys, [&](int e) { return s->rows[e]; });
+}
+
+// NN and NT layouts with many short groups: the groups by descending tile height, so that every
+// round of tiles is made of equal ones and no workgroup is dealt more than its share of the tall
+// ones.  The tile prefix sums are then counted again, in that order (the first wave, as in
+// build_schedule; the totals do not change).
+template <int LAYOUT, int BM, int BN>
+__device__ __forceinline__ void order_groups_by_height(Sched* s, const GmmParams& p, uint64_t* keys) {
+  const int E = p.num_groups;
+  order_groups(s, E, keys, [&](int e) {
+    const int rows = s->rows[e];
+    return rows > 0 ? group_tiles<LAYOUT, BM, BN>(rows, p.hidden_in, p.hidden_out, p.flags).height : 0;
+  });
+  const int lane = threadIdx.x;
+  if (lane < 64) {
+    const int per = (E + 63) >> 6;
+    const int q0 = lane * per;
+    int tsum = 0, rsum = 0;
+    for (int i = 0; i < per; ++i) {
+      const int q = q0 + i;
+      if (q < E) {
+        const GroupTiles g = group_tiles<LAYOUT, BM, BN>(s->rows[s->order[q]], p.hidden_in, p.hidden_out, p.flags);
+        tsum += g.main_rows * g.tiles_n;
+        rsum += g.runt * g.tiles_n;
+      }
+    }
+    int tincl = tsum, rincl = rsum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(tincl, d);
+      const int o2 = __shfl_up(rincl, d);
+      if (lane >= d) {
+        tincl += o;
+        rincl += o2;
+      }
+    }
+    int trun = tincl - tsum, rrun = rincl - rsum;
+    for (int i = 0; i < per; ++i) {
+      const int q = q0 + i;
+      if (q < E) {
+        s->tile_start[q] = trun;
+        s->runt_start[q] = rrun;
+        const GroupTiles g = group_tiles<LAYOUT, BM, BN>(s->rows[s->order[q]], p.hidden_in, p.hidden_out, p.flags);
+        trun += g.main_rows * g.tiles_n;
+        rrun += g.runt * g.tiles_n;
+      }
+    }
+  }
   __syncthreads();
 }
 
@@ -516,10 +579,15 @@ __device__ __forceinline__ void tile_coords(int u, int tiles_m, int tiles_n, int
 template <int LAYOUT, int BM, int BN>
 __global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSizes hs) {
   __shared__ Sched s;
-  __shared__ uint64_t sort_keys[LAYOUT == kTN ? kMaxGroups : 1];
+  __shared__ uint64_t sort_keys[kMaxGroups];
   build_schedule<LAYOUT, BM, BN>(&s, p, hs);
   __syncthreads();
-  if (LAYOUT == kTN) order_groups_by_depth(&s, p.num_groups, sort_keys);
+  const bool ordered = LAYOUT == kTN || (p.flags & kFlagByHeight) != 0;
+  if (LAYOUT == kTN) {
+    order_groups_by_depth(&s, p.num_groups, sort_keys);
+  } else if (ordered) {
+    order_groups_by_height<LAYOUT, BM, BN>(&s, p, sort_keys);
+  }
   for (int e = threadIdx.x; e < p.num_groups; e += 64) {
     const GroupGeom g = group_geometry<LAYOUT>(p, p.first_group + e, s.row_start[e], s.rows[e]);
     const GroupTiles gt = group_tiles<LAYOUT, BM, BN>(s.rows[e], p.hidden_in, p.hidden_out, p.flags);
@@ -534,14 +602,14 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSize
     row[7] = g.b_off;
     row[8] = g.c_off;
     int position = e;   // where the group's tiles stand in the order they are handed out
-    if (LAYOUT == kTN) {
+    if (ordered) {
       for (int q = 0; q < p.num_groups; ++q)
         if (s.order[q] == e) position = q;
     }
     row[9] = s.tile_start[position];
     row[10] = gt.tiles_m * gt.tiles_n;
     row[11] = s.rows[e];
-    row[12] = s.tile_start[p.num_groups] + s.runt_start[e];
+    row[12] = s.tile_start[p.num_groups] + s.runt_start[position];
     row[13] = gt.runt * gt.tiles_n;
   }
 }
@@ -986,9 +1054,11 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
     while (t >= uniform(sched->runt_start[cur.e + 1])) ++cur.e;
     u = t - uniform(sched->runt_start[cur.e]);
   }
-  // (weight-gradient layout: the cursor walks positions of the descending-depth order; all groups
-  // have the same number of tiles there, so the tile prefix sums serve positions as they are)
-  const int e = LAYOUT == kTN ? uniform((int)sched->order[cur.e]) : cur.e;
+  // (the cursor walks positions of the order the groups are handed out in.  Weight-gradient layout:
+  // all groups have the same number of tiles, so the tile prefix sums serve positions as they are;
+  // by tile height: the prefix sums were counted in that order)
+  const bool ordered = LAYOUT == kTN || (p.flags & kFlagByHeight) != 0;
+  const int e = ordered ? uniform((int)sched->order[cur.e]) : cur.e;
   // read through the first lane: everything derived from these stays in scalar registers
   const int rows = uniform(sched->rows[e]);
   ti.g = group_geometry<LAYOUT>(p, p.first_group + e, uniform(sched->row_start[e]), rows);
@@ -1078,7 +1148,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   Sched* sched = reinterpret_cast<Sched*>(smem + Cfg::SCHED_OFFSET);
   build_schedule<LAYOUT, BM, BNS>(sched, p, hs);
   __syncthreads();
-  if constexpr (LAYOUT == kTN) order_groups_by_depth(sched, p.num_groups, reinterpret_cast<uint64_t*>(smem));
+  if constexpr (LAYOUT == kTN) {
+    order_groups_by_depth(sched, p.num_groups, reinterpret_cast<uint64_t*>(smem));
+  } else {
+    if (p.flags & kFlagByHeight) order_groups_by_height<LAYOUT, BM, BNS>(sched, p, reinterpret_cast<uint64_t*>(smem));
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);

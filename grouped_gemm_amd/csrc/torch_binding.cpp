@@ -308,6 +308,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.attr("status_rows_past_end") = GG_STATUS_ROWS_PAST_END;
   m.def("gmm_with_flags", &GroupedGemmWithFlags, "gmm with GG_FLAG_* bits (testing).");
   m.attr("flag_whole_tiles") = GG_FLAG_WHOLE_TILES;
+  m.attr("flag_group_order") = GG_FLAG_GROUP_ORDER;
   m.def("accumulate_weight_gradient", &AccumulateWeightGradient,
         "c (fp32) += per expert a_e^T @ b_e.");
   m.def("debug_schedule", &DebugSchedule, "Per-group table derived by the on-device scheduler.");

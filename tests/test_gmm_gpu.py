@@ -473,6 +473,34 @@ def test_c_abi_without_workspace_cuts_rows_bit_exactly(oracle):
         check(c1, oracle.gmm_loop(a.cpu(), b.cpu(), bs), f"case {idx}")
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_tiles_by_height_against_group_order(ops, oracle, trans_b):
+    # Many short groups of unequal tile heights: their tiles are handed out by descending tile
+    # height (see test_schedule_bit_exact for the order itself).  Every tile is computed as it
+    # would be in group order (shallow products: no depth pieces), so the outputs are equal bit for
+    # bit to those of GG_FLAG_GROUP_ORDER, and right against the oracle.  256 groups take the
+    # counting path of the ranking, 300 with empty ones the sorting path; device- and host-resident sizes.
+    cases = [([200 + (37 * i) % 180 for i in range(256)], 256, 1024),
+             ([0 if i % 7 == 0 else 100 + (53 * i) % 400 for i in range(300)], 192, 1032)]
+    for idx, (sizes, hin, hout) in enumerate(cases):
+        _announce("tiles by height", trans_b, len(sizes), hin, hout)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        assert _handed_out_by_height(len(sizes), t, -(-hout // 256), 256)
+        g = torch.Generator().manual_seed(40 + idx)
+        a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
+        b = (torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g) * hin ** -0.5).to(torch.bfloat16)
+        da, db = a.cuda(), b.cuda()
+        by_height = torch.full((t + 1, hout), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.backend.backend.gmm(da, db, by_height[:t], bs.cuda() if idx == 0 else bs, False, trans_b)
+        in_order = torch.full((t + 1, hout), 7.0, dtype=torch.bfloat16, device="cuda")
+        ops.backend.backend.gmm_with_flags(da, db, in_order[:t], bs.cuda(), False, trans_b,
+                                           ops.backend.backend.flag_group_order)
+        assert torch.equal(by_height, in_order)
+        assert bool((by_height[t] == 7.0).all())
+        check(by_height[:t], oracle.gmm_loop(a, b, bs, trans_b=trans_b), f"case {idx}")
+
+
 # ----------------------------------------------------------------- schedule, bit-exact
 
 SCHED_CASES = [
@@ -482,7 +510,19 @@ SCHED_CASES = [
     ([256] * 256, 7168, 2048),          # b offsets pass 2**31 elements
     ([1] * 512, 8, 8),
     ([70000, 0, 3, 70000], 2048, 1408),
+    # many short groups of unequal tile heights: handed out by tile height (NN and NT); 300 of
+    # them, with empty ones, take the sorting path of the ranking, 256 the counting one
+    ([200 + (37 * i) % 180 for i in range(256)], 7168, 2048),
+    ([0 if i % 7 == 0 else 100 + (53 * i) % 400 for i in range(300)], 512, 1024),
 ]
+
+
+def _handed_out_by_height(num_groups, tokens, tiles_n, bm):
+    # the library's rule (gmm_api.hip, order_by_height): many groups, short on average, and enough
+    # tiles for several rounds
+    grid = torch.cuda.get_device_properties(0).multi_processor_count
+    return (num_groups >= 32 and tokens < 512 * num_groups and
+            (tokens // bm + num_groups // 2) * tiles_n >= 4 * grid)
 
 
 @pytest.mark.parametrize("sizes,hin,hout", SCHED_CASES)
@@ -510,15 +550,31 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
         by_position = np.argsort(got[:, 9], kind="stable")
         assert sorted(by_position.tolist()) == list(range(len(sizes)))
         assert (np.diff(np.array(sizes)[by_position]) <= 0).all()
-    else:
-        assert np.array_equal(got[:, 9], np.cumsum(first_class) - first_class)
-    assert np.array_equal(got[:, 12], first_class.sum() + np.cumsum(got[:, 13]) - got[:, 13])
-    assert np.array_equal(got[:, 11], np.array(sizes))
     lib = ctypes.CDLL(os.path.join(ROOT, "grouped_gemm_amd", "libgrouped_gemm_hip.so"))
     bm, bn, bk = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     lib.gg_tile_shape(ctypes.c_int64(len(sizes)), ctypes.c_int64(tokens), int(trans_a), int(trans_b),
                       ctypes.byref(bm), ctypes.byref(bn), ctypes.byref(bk))
     m, n = got[:, 0], got[:, 1]
+    if not trans_a:
+        # NN and NT: in group order, or, for many short groups, by descending tile height, groups
+        # of equal height in their own order; both prefix sums count in that order
+        order = np.arange(len(sizes))
+        if _handed_out_by_height(len(sizes), tokens, -(-hout // bn.value), bm.value):
+            rows = np.array(sizes)
+            tile_rows = -(-rows // bm.value)
+            heights = np.where(rows > 0, -(-(-(-rows // np.maximum(tile_rows, 1))) // 32) * 32, 0)
+            order = np.argsort(-heights, kind="stable")
+            if len(set(heights.tolist())) > 2:
+                assert not np.array_equal(order, np.arange(len(sizes))), "the case should exercise the order"
+        want_first = np.empty(len(sizes), dtype=np.int64)
+        want_first[order] = (np.cumsum(first_class[order]) - first_class[order])
+        assert np.array_equal(got[:, 9], want_first)
+        want_runt = np.empty(len(sizes), dtype=np.int64)
+        want_runt[order] = first_class.sum() + np.cumsum(got[order, 13]) - got[order, 13]
+        assert np.array_equal(got[:, 12], want_runt)
+    else:
+        assert np.array_equal(got[:, 12], first_class.sum() + np.cumsum(got[:, 13]) - got[:, 13])
+    assert np.array_equal(got[:, 11], np.array(sizes))
     assert np.array_equal(got[:, 10], -(-m // bm.value) * -(-n // bn.value))
     # a runt row is the last tile row of a group of at least two, at most half as many 32-row
     # blocks tall as the others
