@@ -91,20 +91,22 @@ bool use_short_shape(int64_t num_groups, int64_t tokens, int trans_a) {
   return !trans_a && num_groups > 0 && tokens < (int64_t)kShortBelow * num_groups;
 }
 
-// NN and NT layouts: whether the groups' tiles are handed out by descending tile height instead
-// of in group order.  With many groups of about one tile row each (some one tile of up to 256 rows,
-// some two of 130-160), tiles dealt in group order give some workgroups more than their share of
-// the tall ones; by height every round is made of equal tiles.  Measured by permuting the groups:
-// 256 groups of about 256 rows (7168 -> 2048, b stored transposed) 2.09 -> 2.00 ms, b as stored
-// -0.5 %; 64 groups of 768 rows on average +1.3 %; 8 groups of 4096 rows unchanged.  Small calls
-// skip the second ranking pass (1-2 us).
-constexpr int kByHeightGroups = 32;        // at least this many groups
-constexpr int kByHeightRowsBelow = 512;    // ... of fewer rows than this on average
-constexpr int kByHeightRounds = 4;         // ... and at least this many rounds of tiles
+// NN and NT layouts: whether the groups' tiles are handed out by ascending number of tile rows
+// instead of in group order (the kernel still keeps the group order if it finds a group of more
+// than 8 tile rows).  Where group sizes straddle a multiple of the tile height, groups of k and of
+// k + 1 tile rows alternate at random; with equal groups side by side the launch is faster.
+// Measured by permuting the groups, Poisson sizes, 7168 -> 2048, b stored transposed / as stored:
+// 256 groups around 256 rows -3.2 / -2.3 %, 96 around 256 -4.8 / -3.6 %, 128 around 512 -1.8 /
+// -2.2 %, around 768 -3.3 / -3.4 %, 64 around 1024 -1.2 / -1.6 %; around 128, 200, 320, 384, 640,
+// 1536, 2048 rows within +-0.7 %; Zipf sizes with groups of up to 57 tile rows +0.8 / +1.7 %
+// (hence the kernel's guard).  Small calls skip the second ranking pass (1-2 us).
+constexpr int kByTileRowsGroups = 32;         // at least this many groups
+constexpr int kByTileRowsRowsBelow = 2048;    // ... of fewer rows than this on average
+constexpr int kByTileRowsRounds = 4;          // ... and at least this many rounds of tiles
 
-bool order_by_height(int64_t num_groups, int64_t tokens, int64_t tiles_n, int bm, int grid) {
-  return num_groups >= kByHeightGroups && tokens < (int64_t)kByHeightRowsBelow * num_groups &&
-         (tokens / bm + num_groups / 2) * tiles_n >= (int64_t)kByHeightRounds * grid;
+bool order_by_tile_rows(int64_t num_groups, int64_t tokens, int64_t tiles_n, int bm, int grid) {
+  return num_groups >= kByTileRowsGroups && tokens < (int64_t)kByTileRowsRowsBelow * num_groups &&
+         (tokens / bm + num_groups / 2) * tiles_n >= (int64_t)kByTileRowsRounds * grid;
 }
 
 // Scratch of gg_gmm_no_alloc: the workspace of gg_gmm (arrival counters, then partial tiles) as a
@@ -417,10 +419,10 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     }
     if (tiles >= (int64_t(1) << 31)) return fail(GG_ELIMIT, "too many output tiles for one launch");
     if (tiles == 0) continue;
-    p.flags &= ~gg::kFlagByHeight;
-    if (!generic && !trans_a && !(p.flags & gg::kFlagGroupOrder) && count >= kByHeightGroups &&
-        order_by_height(num_groups, tokens, tiles_n, bm, info.cus))
-      p.flags |= gg::kFlagByHeight;
+    p.flags &= ~gg::kFlagByTileRows;
+    if (!generic && !trans_a && !(p.flags & gg::kFlagGroupOrder) && count >= kByTileRowsGroups &&
+        order_by_tile_rows(num_groups, tokens, tiles_n, bm, info.cus))
+      p.flags |= gg::kFlagByTileRows;
     // the full grid also for few tiles: the last round's tiles may be cut into pieces for
     // the workgroups that would otherwise idle
     if (generic) {
@@ -554,9 +556,9 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   const bool short_shape = use_short_shape(num_groups, tokens, trans_a);
   {
     const int bm = short_shape ? Short::BM : Wide::BM, bn = short_shape ? Short::BN : Wide::BN;
-    if (!trans_a && num_groups >= kByHeightGroups &&
-        order_by_height(num_groups, tokens, (hidden_out + bn - 1) / bn, bm, info.cus))
-      p.flags |= gg::kFlagByHeight;
+    if (!trans_a && num_groups >= kByTileRowsGroups &&
+        order_by_tile_rows(num_groups, tokens, (hidden_out + bn - 1) / bn, bm, info.cus))
+      p.flags |= gg::kFlagByTileRows;
   }
   gg::HostSizes hs;
   if (batch_sizes_on_device) {

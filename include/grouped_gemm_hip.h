@@ -61,7 +61,7 @@ extern "C" {
 #define GG_FLAG_WHOLE_TILES 1   /* never cut the tiles of the last round into pieces */
 #define GG_FLAG_ONE_CLASS 2     /* hand out a tall group's short last tile row in place, not after all other tiles */
 #define GG_FLAG_ROW_PIECES 4    /* ignore the workspace: cut the last round's tiles along the rows only */
-#define GG_FLAG_GROUP_ORDER 8   /* hand out the groups' tiles in group order, also where the library would hand them out by tile height (many short groups, trans_a = 0) */
+#define GG_FLAG_GROUP_ORDER 8   /* hand out the groups' tiles in group order, also where the library would hand them out by their number of tile rows (many short groups, trans_a = 0) */
 
 /*
  * One-time set-up for the current device: checks that it is a gfx950 and raises the LDS limit
