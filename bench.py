@@ -34,10 +34,10 @@ PEAK_HBM_GBPS = 8000.0
 # the hash below (kernel_sources_sha16), and is reported only while the sources still have that
 # hash; the summary under profiles/ holds the figures, the commands and the commit.
 _TRAFFIC_KERNEL_SOURCES = ("gmm_kernel.hpp", "gmm_api.hip", "gmm_variants.hpp", "gmm_variants.def", "gmm_variant.hip")
-_TRAFFIC_KERNEL_SHA16 = "ccc3f41735a7be25"
+_TRAFFIC_KERNEL_SHA16 = "852f504fdd8fbe49"
 _TRAFFIC_SOURCE = ("profiles/gmm_kernel_mixtral_w1_hbm_traffic.md and profiles/gmm_kernel_configs_3_4_5_stats_and_traffic.md "
                    "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources sha16 " + _TRAFFIC_KERNEL_SHA16 +
-                   ", commit 97b589b; profiled once, not in this run)")
+                   ", commit bb55182; profiled once, not in this run)")
 
 
 def kernel_sources_sha16():
@@ -55,10 +55,10 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    2: {"fwd": _traffic(4048330, 917552), "agrad": _traffic(3327810, 290043), "bgrad": _traffic(2752750, 917526)},
-    3: {"fwd": _traffic(444298, 135176)},
-    4: {"bgrad": _traffic(2752750, 917513)},
-    5: {"fwd": _traffic(4332400, 262156), "agrad": _traffic(5438120, 917511), "bgrad": _traffic(1851750, 7343380)},
+    2: {"fwd": _traffic(4045360, 917534), "agrad": _traffic(3324540, 289918), "bgrad": _traffic(2760500, 917514)},
+    3: {"fwd": _traffic(430485, 135193)},
+    4: {"bgrad": _traffic(2753450, 917527)},
+    5: {"fwd": _traffic(4149630, 262175), "agrad": _traffic(4849680, 917550), "bgrad": _traffic(1851720, 7344320)},
 }
 
 
