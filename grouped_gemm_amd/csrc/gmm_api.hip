@@ -488,8 +488,9 @@ uint64_t gg_workspace_bytes_for(const gg_gmm_args* args) {
   if (g.flags & (GG_FLAG_WHOLE_TILES | GG_FLAG_ROW_PIECES)) return 0;
   {
     const int64_t slice = r.elem_bytes == 1 ? 2 * gg::BK : gg::BK;   // depth elements per slice
-    // (weight-gradient layout: the depth is the group's row count, taken as the average)
-    const int64_t depth = g.trans_a ? g.tokens / (g.num_groups > 0 ? g.num_groups : 1) : g.hidden_in;
+    // (weight-gradient layout: the depth is a group's row count, and one group may hold all rows:
+    // the kernel cuts the tiles of groups much deeper than the rest, plan_deep_tiles)
+    const int64_t depth = g.trans_a ? g.tokens : g.hidden_in;
     if ((depth + slice - 1) / slice < 2 * gg::kMinSlicesPerPiece) return 0;
   }
   return GG_WORKSPACE_BYTES;

@@ -169,6 +169,12 @@ struct Sched {
   int32_t tile_start[kMaxGroups + 1];  // exclusive prefix sum of the first class's tiles
   int32_t runt_start[kMaxGroups + 1];  // exclusive prefix sum of the runt rows' tiles
   int32_t arrived;                     // broadcast slot for the arrival count of a depth piece
+  int32_t fix_tile[24];                // the tile whose depth pieces this workgroup adds up after its last tile
+  // Weight-gradient layout (plan_deep_tiles): the first front_tiles tiles, the deepest ones, are
+  // cut along the depth into front_pieces pieces each; tile indices 0 .. front_tiles *
+  // front_pieces - 1 name those pieces, the tiles behind follow whole, and the last round is not
+  // cut.  (Kept here, not in registers: the tile loop has no scalar registers to spare.)
+  int32_t front_tiles, front_pieces;
   // order[q] is the group whose tiles are handed out q-th.  Weight-gradient layout: by descending
   // depth.  Every group has the same number of tiles there and a tile's cost is its group's depth,
   // so the deepest groups go first and the shallow ones fill the end of the launch: what the
@@ -409,6 +415,8 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
     }
   }
   if (lane == 63) {
+    s->front_tiles = 0;
+    s->front_pieces = 1;
     s->row_start[E] = (int)(run < p.tokens ? run : p.tokens);
     s->tile_start[E] = tincl;
     s->runt_start[E] = rincl;
@@ -492,6 +500,42 @@ __device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, 
     return;
   }
   order_groups(s, num_groups, keys, [&](int e) { return s->rows[e]; });
+}
+
+// Weight-gradient layout with a workspace, after order_groups_by_depth: tiles go out by descending
+// depth, one workgroup each, so a group much deeper than the others sets the length of the launch
+// however its tiles are dealt (Zipf depths: the deepest tile 227 slices, 144 slices of work per
+// workgroup).  When the deepest tile is longer than a workgroup's even share of all depth slices,
+// the tiles deeper than half that share (and deep enough to pay for their fix-up) are cut into 2
+// or 4 depth pieces, which are handed out first, one per workgroup.  Run by every thread; the
+// same answer in each.
+__device__ __forceinline__ void plan_deep_tiles(Sched* s, const GmmParams& p, int grid, int bk, TailPlan* plan) {
+  const int E = p.num_groups;
+  const int tiles = s->tile_start[E];
+  if (E == 0 || tiles == 0 || p.ws_slots <= 0 || (p.flags & (kFlagWholeTiles | kFlagRowPieces))) return;
+  const int per_group = tiles / E;   // (every group has the same number of tiles in this layout)
+  int64_t slices = 0;
+  for (int j = 0; j < E; ++j) slices += (s->rows[j] + bk - 1) / bk;   // (broadcast reads)
+  const int64_t share = slices * per_group / grid;
+  const int deepest = (s->rows[s->order[0]] + bk - 1) / bk;
+  const int pieces = deepest >= 4 * kMinSlicesPerPiece ? 4 : (deepest >= 2 * kMinSlicesPerPiece ? 2 : 0);
+  if (pieces == 0 || deepest <= share) return;
+  int most = grid / pieces;
+  most = most < p.ws_slots / pieces ? most : p.ws_slots / pieces;
+  most = most < kWsCounterBytes / 4 ? most : kWsCounterBytes / 4;
+  int front = 0;
+  for (int q = 0; q < E && front < most; ++q) {
+    const int depth = (s->rows[s->order[q]] + bk - 1) / bk;
+    if (2 * (int64_t)depth <= share || depth < pieces * kMinSlicesPerPiece) break;
+    front += per_group;
+  }
+  front = front < most ? front : most;
+  if (front == 0) return;
+  s->front_tiles = front;     // (every thread writes the same two values, and reads its own wave's)
+  s->front_pieces = pieces;
+  plan->pieces = 1;   // the last round stays whole: a workgroup has at most one tile to fix
+  plan->by_depth = true;
+  plan->main_tiles = plan->total = front * pieces + (tiles - front);
 }
 
 // NN and NT layouts with many short groups: the groups by ascending number of tile rows, groups
@@ -1060,7 +1104,20 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
     return ti;
   }
   int piece = -1;
-  if (t >= plan.main_tiles) {
+  int pieces = plan.pieces;
+  const int front_tiles = LAYOUT == kTN ? uniform(sched->front_tiles) : 0;
+  if (front_tiles > 0) {
+    const int front_pieces = uniform(sched->front_pieces);
+    const int cut = front_tiles * front_pieces;
+    if (t < cut) {
+      pieces = front_pieces;
+      piece = t % pieces;
+      ti.rank = t / pieces;
+      t = ti.rank;
+    } else {
+      t = t - cut + front_tiles;
+    }
+  } else if (t >= plan.main_tiles) {
     const int r = t - plan.main_tiles;
     piece = r % plan.pieces;
     ti.rank = r / plan.pieces;
@@ -1104,8 +1161,8 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   ti.nk = nk < 1 ? 1 : nk;
   if (piece >= 0 && plan.by_depth) {
     // this piece's share of the depth slices; a piece without slices contributes zeros
-    const int first = piece * ti.nk / plan.pieces, last = (piece + 1) * ti.nk / plan.pieces;
-    ti.pieces = plan.pieces;
+    const int first = piece * ti.nk / pieces, last = (piece + 1) * ti.nk / pieces;
+    ti.pieces = pieces;
     ti.piece = piece;
     ti.k0 = first;
     ti.nk = last - first;
@@ -1117,7 +1174,7 @@ __device__ __forceinline__ TileInfo find_tile(const Sched* sched, const GmmParam
   } else if (piece >= 0) {
     // this piece's share of the tile's 32-row blocks; a piece past the rows is an empty tile
     const int all = (ti.rows_valid + 31) / 32;
-    const int per = (all + plan.pieces - 1) / plan.pieces;
+    const int per = (all + pieces - 1) / pieces;
     const int skip = piece * per * 32;
     ti.m0 += skip;
     ti.rows_valid = min(per * 32, ti.rows_valid - skip);
@@ -1196,6 +1253,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       uniform(sched->tile_start[p.num_groups]) + uniform(sched->runt_start[p.num_groups]),
       (int)gridDim.x, p, BK_ELEMS);
   if constexpr (!DEPTH_PIECES) plan.by_depth = false;   // (known at compile time: no depth-piece code is kept)
+  if constexpr (LAYOUT == kTN && DEPTH_PIECES) {
+    plan_deep_tiles(sched, p, (int)gridDim.x, BK_ELEMS, &plan);
+    plan.pieces = uniform(plan.pieces), plan.main_tiles = uniform(plan.main_tiles), plan.total = uniform(plan.total);
+  }
   const int total_tiles = plan.total;
 
   // Workgroups are dealt to the 8 XCDs round-robin; give each XCD a contiguous run of
@@ -1359,9 +1420,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // Partial tile of depth piece `piece` of the tile `ti` names, as this thread sees it: a lane's
   // 16-byte group (i, j, q) sits at ((i * NB + j) * 4 + q) * NT + thread, so one instruction of a
   // wave moves 1 KiB of consecutive bytes.
-  auto partial_slot = [&](int piece) {
+  auto partial_slot = [&](const TileInfo& tile, int piece) {
     return reinterpret_cast<float*>(p.workspace + kWsCounterBytes) +
-           (int64_t)(ti.rank * ti.pieces + piece) * (BM * BN) + threadIdx.x * 4;
+           (int64_t)(tile.rank * tile.pieces + piece) * (BM * BN) + threadIdx.x * 4;
   };
   bool fix_pending = false;   // this workgroup's depth piece was the last of its tile to arrive
 
@@ -1449,7 +1510,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
     // count the arrival.  The piece that arrives last adds the partial tiles up and stores the
     // sum, after the tile loop (fix_up below), where no accumulator is live any more.
     if (DEPTH_PIECES && ti.pieces > 1) {
-      float* mine = partial_slot(ti.piece);
+      float* mine = partial_slot(ti, ti.piece);
 #pragma unroll
       for (int i = 0; i < ML; ++i)
 #pragma unroll
@@ -1464,6 +1525,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       if (threadIdx.x == 0) sched->arrived = atomicAdd(reinterpret_cast<int*>(p.workspace) + ti.rank, 1);
       block_barrier();
       fix_pending = uniform(sched->arrived) == ti.pieces - 1;
+      if (fix_pending) {
+        // Keep the tile's description for the fix-up after the tile loop (a piece of the last
+        // round is this workgroup's last tile, one of a deep tile its first): copied from the
+        // slot of the tile ring it was read from, which the fetch cursor, at most two tiles
+        // ahead, has not reached again.  (Packing it from registers would keep every field live
+        // through the depth loop, which has no scalar registers to spare.)
+        static_assert(sizeof(sched->fix_tile) == kTileInfoDwords * 4 && kTileInfoDwords <= 64, "");
+        if (threadIdx.x < kTileInfoDwords)
+          sched->fix_tile[threadIdx.x] = tile_ring[(tile_n % Cfg::TILE_RING_SLOTS) * kTileInfoDwords + threadIdx.x];
+      }
       return;
     }
 
@@ -1687,28 +1758,33 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   }
   wait_vmcnt<0>();   // the zero-filling fetches past the last tile still write LDS
 
-  // Fix-up of a tile that was cut along the depth.  Pieces exist in the last round only, so a
-  // piece is its workgroup's last tile and `ti` still names it.  The partial tiles are added up
-  // in piece order, two per step (their count is even), whichever piece does the adding, so the
-  // result does not depend on timing.  One block row of 32 rows at a time: NB * 4 groups of 16
-  // bytes per lane and piece.
+  // Fix-up of a tile that was cut along the depth: the tile this workgroup left in
+  // Sched::fix_tile when its piece arrived last (a workgroup has at most one).  The partial tiles
+  // are added up in piece order, two per step (their count is even), whichever piece does the
+  // adding, so the result does not depend on timing.  One block row of 32 rows at a time: NB * 4
+  // groups of 16 bytes per lane and piece.
   if (DEPTH_PIECES && fix_pending) {
+    __syncthreads();   // (the description was written by the first thread)
+    int32_t words[kTileInfoDwords];
+#pragma unroll
+    for (int i = 0; i < kTileInfoDwords; ++i) words[i] = sched->fix_tile[i];
+    const TileInfo ft = unpack_tile(words);
     __threadfence();   // the other pieces' partial tiles are visible to this workgroup
-    if (threadIdx.x == 0) reinterpret_cast<int*>(p.workspace)[ti.rank] = 0;   // leave the counters as they were found
+    if (threadIdx.x == 0) reinterpret_cast<int*>(p.workspace)[ft.rank] = 0;   // leave the counters as they were found
     constexpr int CE = ACC_F32 ? 4 : 2;   // bytes per element of c
-    const char* cbase = p.c + (ti.g.c_off + (int64_t)ti.m0 * ti.g.n) * CE;
-    const uint32_t cbytes = ti.rows_valid > 0 ? (uint32_t)(ti.rows_valid * ti.g.n) * (uint32_t)CE : 0u;
+    const char* cbase = p.c + (ft.g.c_off + (int64_t)ft.m0 * ft.g.n) * CE;
+    const uint32_t cbytes = ft.rows_valid > 0 ? (uint32_t)(ft.rows_valid * ft.g.n) * (uint32_t)CE : 0u;
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(cbase, cbytes);
-    const int live = LAYOUT == kTN ? MB : (ti.blocks - wm + WAVES_M - 1) / WAVES_M;
+    const int live = LAYOUT == kTN ? MB : (ft.blocks - wm + WAVES_M - 1) / WAVES_M;
     for (int i = 0; i < live; ++i) {
       f32x4 sum[NB][4];
 #pragma unroll
       for (int j = 0; j < NB; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) sum[j][q] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      for (int piece = 0; piece < ti.pieces; piece += 2) {
-        const float* from0 = partial_slot(piece) + (i * NB * 4) * (NT * 4);
-        const float* from1 = partial_slot(piece + 1) + (i * NB * 4) * (NT * 4);
+      for (int piece = 0; piece < ft.pieces; piece += 2) {
+        const float* from0 = partial_slot(ft, piece) + (i * NB * 4) * (NT * 4);
+        const float* from1 = partial_slot(ft, piece + 1) + (i * NB * 4) * (NT * 4);
         f32x4 v0[NB][4], v1[NB][4];
 #pragma unroll
         for (int j = 0; j < NB; ++j)
@@ -1728,8 +1804,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
       for (int j = 0; j < NB; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int col = ti.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
-          const uint32_t off = col < ti.g.n ? (uint32_t)(row * ti.g.n + col) * (uint32_t)CE : kOutOfRange;
+          const int col = ft.n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+          const uint32_t off = col < ft.g.n ? (uint32_t)(row * ft.g.n + col) * (uint32_t)CE : kOutOfRange;
           if constexpr (ACC_F32) {
             const f32x4 old = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rc, off, 0, 0));
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, old + sum[j][q]), rc, off, 0, 0);

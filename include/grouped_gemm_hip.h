@@ -171,10 +171,13 @@ int gg_gmm_bf16_acc_f32(const void* a, const void* b, float* c, const int64_t* b
  *   workspace, workspace_bytes
  *                 Device memory the call may use for partial results, or NULL.  When the last
  *                 round of the persistent grid is at most half full, each of its tiles is cut
- *                 into 2 to 8 pieces along the depth; a piece adds up its depth slices into an
+ *                 into 2 or 4 pieces along the depth; a piece adds up its depth slices into an
  *                 fp32 partial tile in the workspace, and the piece that finishes last sums the
  *                 partial tiles in piece order and stores the result, so the output does not
- *                 depend on timing.  The first 4096 bytes (arrival counters) must be zero
+ *                 depend on timing.  With trans_a = 1, when a group is so much deeper than the
+ *                 rest that its tiles alone would set the length of the launch, the tiles of
+ *                 such groups are cut the same way and handed out first (instead of the last
+ *                 round's).  The first 4096 bytes (arrival counters) must be zero
  *                 before the first call and are zero again after every call; the rest needs no
  *                 initialisation.  GG_WORKSPACE_BYTES serves every call; a smaller workspace
  *                 (at least 4096 + one 256 KiB tile) serves fewer pieces; 256-byte aligned.
@@ -217,7 +220,7 @@ int gg_gmm(const gg_gmm_args* args);
  * Bytes of workspace the call described by `args` can make use of: 0 when no launch of it ever
  * cuts tiles along the depth (general kernels, row indices, the SwiGLU epilogue, or a product too
  * shallow for depth pieces to pay: fewer than 96 depth slices of 64 two-byte or 128 one-byte
- * elements, the depth of the trans_a layout being the average rows per group),
+ * elements, the depth of the trans_a layout being what one group could hold, i.e. all rows),
  * GG_WORKSPACE_BYTES otherwise.  Looks at the sizes, flags
  * and pointers' alignment only; args->workspace is ignored.  A caller that keeps workspaces
  * (one per stream) need not allocate one for calls this returns 0 for.  No counterpart in the

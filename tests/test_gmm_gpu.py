@@ -448,6 +448,66 @@ def test_last_round_pieces_against_whole_tiles(ops, oracle, layout):
         assert torch.equal(cut, _gmm_flags(ops, a, b, dev_bs, 0, trans_a, trans_b))
 
 
+def test_deep_groups_of_a_weight_gradient_are_cut_first(oracle):
+    # Weight gradient with one or two groups much deeper than the rest: their tiles would set the
+    # length of the launch, so they are cut along the depth into 2 or 4 pieces that go out first,
+    # one per workgroup; whichever piece arrives last adds the partial tiles up, after its
+    # workgroup's other tiles.  Through the C ABI with a workspace of the test's own: the cut
+    # leaves partial tiles in it (exactly as many as the plan says) and the arrival counters at
+    # zero.  Against the oracle, against whole tiles (fp32 summation order apart), the same bits
+    # on every call, zero-row groups all zero.
+    lib = _c_abi()
+    cases = [  # sizes, hidden_in, hidden_out, tiles cut, pieces each
+        ([14000, 300, 200, 0, 150, 6500, 100, 120], 264, 520, 6, 4),   # the group of 6500 rows is too shallow for 4 pieces
+        ([7000, 100, 6800], 136, 264, 4, 2),                           # two deep groups, 2 pieces
+        ([64] * 50 + [20000] + [64] * 50, 256, 256, 1, 4),
+        ([13000, 50, 12800], 1024, 2048, 64, 4),                       # more deep tiles than a round has room for
+        ([6080, 100, 90], 264, 520, 0, 0),                             # 95 slices: too shallow to pay for a fix-up
+        ([7000, 7000, 7000, 7000], 2048, 4096, 0, 0),                  # deep, but no deeper than a workgroup's share
+    ]
+    slot = 256 * 256
+    for idx, (sizes, hin, hout, cut_tiles, pieces) in enumerate(cases):
+        _announce("deep groups first", sizes if len(sizes) < 10 else len(sizes), hin, hout)
+        g = torch.Generator().manual_seed(300 + idx)
+        bs = torch.tensor(sizes, dtype=torch.int64)
+        t = int(bs.sum())
+        a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
+        b = torch.randn(t, hout, generator=g).to(torch.bfloat16).cuda()
+        dbs = bs.cuda() if idx % 2 else bs
+        shape = (len(sizes), hin, hout)
+        ws = torch.zeros(1024 + 256 * slot, dtype=torch.float32, device="cuda")
+        cut = torch.full(shape, 7.0, dtype=torch.bfloat16, device="cuda")
+        args = _gmm_args(lib, a, b, cut, dbs, bool(idx % 2), t, hin, hout, True, False, workspace=ws)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
+        torch.cuda.synchronize()
+        assert not bool(ws[:1024].any()), "arrival counters left nonzero"
+        # (a launch with fewer tiles than workgroups may also cut its last round: the deep-group
+        # cut comes instead of that one, so the count below is either the one or the other)
+        used = int((ws[1024:].view(256, slot) != 0).any(dim=1).sum())
+        if cut_tiles:
+            assert used == cut_tiles * pieces, f"case {idx}: {used} partial tiles in the workspace"
+        whole = torch.full(shape, 7.0, dtype=torch.bfloat16, device="cuda")
+        args = _gmm_args(lib, a, b, whole, dbs, bool(idx % 2), t, hin, hout, True, False, workspace=ws, flags=1)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
+        again = torch.full(shape, 7.0, dtype=torch.bfloat16, device="cuda")
+        args = _gmm_args(lib, a, b, again, dbs, bool(idx % 2), t, hin, hout, True, False, workspace=ws)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(cut, again)
+        if hin * hout <= 1024 * 2048:
+            want = oracle.gmm_loop(a.cpu(), b.cpu(), bs, trans_a=True)
+            check(whole, want, f"whole, case {idx}")
+            check(cut, want, f"cut, case {idx}")
+        else:   # at this size the per-expert fp32 product on the GPU stands in for the CPU loop
+            want = torch.stack([a[s:e].float().t() @ b[s:e].float() for s, e in
+                                zip((bs.cumsum(0) - bs).tolist(), bs.cumsum(0).tolist())])
+            check(cut, want, f"cut, case {idx}")
+        assert float((cut.float() - whole.float()).abs().max()) <= 2 ** -7 * float(whole.float().abs().max())
+        for e, rows in enumerate(sizes):
+            if rows == 0:
+                assert not bool(cut[e].any())
+
+
 def test_c_abi_without_workspace_cuts_rows_bit_exactly(oracle):
     # gg_gmm_bf16 brings no workspace: the tiles of the last round are cut along their rows, which
     # leaves the depth order of every output element alone, so the result equals the whole-tile
