@@ -175,6 +175,7 @@ struct Sched {
   // front_pieces - 1 name those pieces, the tiles behind follow whole, and the last round is not
   // cut.  (Kept here, not in registers: the tile loop has no scalar registers to spare.)
   int32_t front_tiles, front_pieces;
+  int32_t most_rows;                   // rows of the largest group
   // order[q] is the group whose tiles are handed out q-th.  Weight-gradient layout: by descending
   // depth.  Every group has the same number of tiles there and a tile's cost is its group's depth,
   // so the deepest groups go first and the shallow ones fill the end of the launch: what the
@@ -414,9 +415,18 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
       rrun += g.runt * g.tiles_n;
     }
   }
+  int most = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) most = rows[i] > most ? rows[i] : most;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    const int o = __shfl_xor(most, d);
+    most = o > most ? o : most;
+  }
   if (lane == 63) {
     s->front_tiles = 0;
     s->front_pieces = 1;
+    s->most_rows = most;
     s->row_start[E] = (int)(run < p.tokens ? run : p.tokens);
     s->tile_start[E] = tincl;
     s->runt_start[E] = rincl;
@@ -440,15 +450,19 @@ __device__ __forceinline__ void order_groups(Sched* s, int num_groups, uint64_t*
   // Up to a few hundred groups it is quicker to count, per group, the groups that go before it
   // (measured equal at 256 groups, 12 us slower than the sort at 512).
   if (num_groups <= 256) {
+    // keys + 1, four to a 16-byte read (the same address in every lane: a broadcast), padded
+    // with zeros, which go before nothing
     uint32_t* key32 = reinterpret_cast<uint32_t*>(keys);
-    for (int e = threadIdx.x; e < num_groups; e += blockDim.x) key32[e] = (uint32_t)key_of(e);
+    const int padded = (num_groups + 3) & ~3;
+    for (int e = threadIdx.x; e < padded; e += blockDim.x) key32[e] = e < num_groups ? (uint32_t)key_of(e) + 1u : 0u;
     __syncthreads();
     for (int e = threadIdx.x; e < num_groups; e += blockDim.x) {
       const uint32_t mine = key32[e];
       int before = 0;
-      for (int j = 0; j < num_groups; ++j) {
-        const uint32_t other = key32[j];   // (the same address in every lane: a broadcast read)
-        before += (other > mine || (other == mine && j < e)) ? 1 : 0;
+      for (int j = 0; j < padded; j += 4) {
+        const u32x4 other = *reinterpret_cast<const u32x4*>(key32 + j);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) before += (other[i] > mine || (other[i] == mine && j + i < e)) ? 1 : 0;
       }
       s->order[before] = (int16_t)e;
     }
@@ -514,10 +528,10 @@ __device__ __forceinline__ void plan_deep_tiles(Sched* s, const GmmParams& p, in
   const int tiles = s->tile_start[E];
   if (E == 0 || tiles == 0 || p.ws_slots <= 0 || (p.flags & (kFlagWholeTiles | kFlagRowPieces))) return;
   const int per_group = tiles / E;   // (every group has the same number of tiles in this layout)
-  int64_t slices = 0;
-  for (int j = 0; j < E; ++j) slices += (s->rows[j] + bk - 1) / bk;   // (broadcast reads)
+  // depth slices of all groups together: their rows, and half a slice per group for the rounding
+  const int64_t slices = ((int64_t)s->row_start[E] - s->row_start[0] + (int64_t)E * (bk / 2)) / bk;
   const int64_t share = slices * per_group / grid;
-  const int deepest = (s->rows[s->order[0]] + bk - 1) / bk;
+  const int deepest = (s->most_rows + bk - 1) / bk;
   const int pieces = deepest >= 4 * kMinSlicesPerPiece ? 4 : (deepest >= 2 * kMinSlicesPerPiece ? 2 : 0);
   if (pieces == 0 || deepest <= share) return;
   int most = grid / pieces;
@@ -551,9 +565,7 @@ constexpr int kMaxTileRowsForOrder = 8;
 template <int LAYOUT, int BM, int BN>
 __device__ __forceinline__ void order_groups_by_tile_rows(Sched* s, const GmmParams& p, uint64_t* keys) {
   const int E = p.num_groups;
-  int most_rows = 0;
-  for (int j = 0; j < E; ++j) most_rows = max(most_rows, s->rows[j]);   // (broadcast reads: the same in every thread)
-  if (most_rows > kMaxTileRowsForOrder * BM) {
+  if (s->most_rows > kMaxTileRowsForOrder * BM) {
     for (int e = threadIdx.x; e < E; e += blockDim.x) s->order[e] = (int16_t)e;
     __syncthreads();
     return;
