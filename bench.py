@@ -34,10 +34,10 @@ PEAK_HBM_GBPS = 8000.0
 # the hash below (kernel_sources_sha16), and is reported only while the sources still have that
 # hash; the summary under profiles/ holds the figures, the commands and the commit.
 _TRAFFIC_KERNEL_SOURCES = ("gmm_kernel.hpp", "gmm_api.hip", "gmm_variants.hpp", "gmm_variants.def", "gmm_variant.hip")
-_TRAFFIC_KERNEL_SHA16 = "5aead35209a9e010"
+_TRAFFIC_KERNEL_SHA16 = "045f884dc1e50d50"
 _TRAFFIC_SOURCE = ("profiles/gmm_kernel_mixtral_w1_hbm_traffic.md and profiles/gmm_kernel_configs_3_4_5_stats_and_traffic.md "
                    "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources sha16 " + _TRAFFIC_KERNEL_SHA16 +
-                   ", commit 52f18d0; profiled once, not in this run)")
+                   ", commit 98af9bb; profiled once, not in this run)")
 
 
 def kernel_sources_sha16():
@@ -55,10 +55,10 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    2: {"fwd": _traffic(4012160, 917547), "agrad": _traffic(3327750, 290011), "bgrad": _traffic(2754780, 917531)},
-    3: {"fwd": _traffic(427725, 135184)},
-    4: {"bgrad": _traffic(2753750, 917526)},
-    5: {"fwd": _traffic(4178330, 262201), "agrad": _traffic(4896200, 917514), "bgrad": _traffic(1851720, 7343790)},
+    2: {"fwd": _traffic(4062210, 917560), "agrad": _traffic(3329380, 290003), "bgrad": _traffic(2756980, 917521)},
+    3: {"fwd": _traffic(422720, 135175)},
+    4: {"bgrad": _traffic(2753160, 917516)},
+    5: {"fwd": _traffic(4207000, 262214), "agrad": _traffic(4800420, 917585), "bgrad": _traffic(1851710, 7344130)},
 }
 
 
