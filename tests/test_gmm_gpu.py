@@ -873,6 +873,39 @@ def test_hip_graph_replay_with_new_device_sizes(ops, oracle):
         check(out, oracle.gmm_loop(a.cpu(), b.cpu(), torch.tensor(new_sizes)), f"replay {new_sizes}")
 
 
+def test_hip_graph_replay_of_a_weight_gradient_with_deep_groups(ops, oracle):
+    # The weight gradient decides inside the kernel, from the sizes it finds, whether the tiles of
+    # a much deeper group are cut along the depth and handed out first (through the binding's
+    # per-stream workspace): one captured launch replays as a balanced launch, as one with the
+    # deep group in the first, the last or a middle place, and as a balanced one again, each equal
+    # to the eager call bit for bit and right against the oracle.
+    hin, hout, t = 264, 520, 16000
+    g = torch.Generator().manual_seed(29)
+    a = torch.randn(t, hin, generator=g).to(torch.bfloat16).cuda()
+    grad = torch.randn(t, hout, generator=g).to(torch.bfloat16).cuda()
+    sizes = torch.tensor([3200] * 5, dtype=torch.int64).cuda()
+    wgrad = torch.empty(5, hin, hout, dtype=torch.bfloat16, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):      # warm-up outside the capture (workspace, first-call attribute setting)
+        ops.backend.gmm(a, grad, sizes, trans_a=True, c=wgrad)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.backend.gmm(a, grad, sizes, trans_a=True, c=wgrad)
+    for new_sizes in ([3200] * 5, [15000, 200, 300, 0, 500], [100, 0, 200, 300, 15400], [0, 500, 14500, 0, 1000],
+                      [7000, 8000, 0, 0, 1000], [3200] * 5):
+        _announce("graph replay, weight gradient", new_sizes)
+        sizes.copy_(torch.tensor(new_sizes, dtype=torch.int64))
+        wgrad.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = ops.backend.gmm(a, grad, sizes, trans_a=True)
+        assert torch.equal(wgrad, eager), new_sizes
+        check(wgrad, oracle.gmm_loop(a.cpu(), grad.cpu(), torch.tensor(new_sizes), trans_a=True), f"replay {new_sizes}")
+
+
 _COLD_CAPTURE = r"""
 import sys, torch
 sys.path.insert(0, sys.argv[1])
