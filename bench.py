@@ -34,10 +34,10 @@ PEAK_HBM_GBPS = 8000.0
 # the hash below (kernel_sources_sha16), and is reported only while the sources still have that
 # hash; the summary under profiles/ holds the figures, the commands and the commit.
 _TRAFFIC_KERNEL_SOURCES = ("gmm_kernel.hpp", "gmm_api.hip", "gmm_variants.hpp", "gmm_variants.def", "gmm_variant.hip")
-_TRAFFIC_KERNEL_SHA16 = "045f884dc1e50d50"
+_TRAFFIC_KERNEL_SHA16 = "8182c52ed2fe41b5"
 _TRAFFIC_SOURCE = ("profiles/gmm_kernel_mixtral_w1_hbm_traffic.md and profiles/gmm_kernel_configs_3_4_5_stats_and_traffic.md "
                    "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources sha16 " + _TRAFFIC_KERNEL_SHA16 +
-                   ", commit 98af9bb; profiled once, not in this run)")
+                   ", commit cb4e047; profiled once, not in this run)")
 
 
 def kernel_sources_sha16():
@@ -55,10 +55,10 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    2: {"fwd": _traffic(4062210, 917560), "agrad": _traffic(3329380, 290003), "bgrad": _traffic(2756980, 917521)},
-    3: {"fwd": _traffic(422720, 135175)},
-    4: {"bgrad": _traffic(2753160, 917516)},
-    5: {"fwd": _traffic(4207000, 262214), "agrad": _traffic(4800420, 917585), "bgrad": _traffic(1851710, 7344130)},
+    2: {"fwd": _traffic(4074460, 917559), "agrad": _traffic(3328030, 290012), "bgrad": _traffic(2757060, 917521)},
+    3: {"fwd": _traffic(434610, 135179)},
+    4: {"bgrad": _traffic(2753720, 917525)},
+    5: {"fwd": _traffic(4241770, 262179), "agrad": _traffic(4985550, 917534), "bgrad": _traffic(1851760, 7344020)},
 }
 
 
