@@ -55,10 +55,10 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    2: {"fwd": _traffic(4074460, 917559), "agrad": _traffic(3328030, 290012), "bgrad": _traffic(2757060, 917521)},
-    3: {"fwd": _traffic(434610, 135179)},
-    4: {"bgrad": _traffic(2753720, 917525)},
-    5: {"fwd": _traffic(4241770, 262179), "agrad": _traffic(4985550, 917534), "bgrad": _traffic(1851760, 7344020)},
+    2: {"fwd": _traffic(4067560, 917548), "agrad": _traffic(3329000, 290034), "bgrad": _traffic(2752940, 917524)},
+    3: {"fwd": _traffic(429810, 135172)},
+    4: {"bgrad": _traffic(2752840, 917520)},
+    5: {"fwd": _traffic(4246760, 262192), "agrad": _traffic(4874290, 917554), "bgrad": _traffic(1851760, 7343680)},
 }
 
 
