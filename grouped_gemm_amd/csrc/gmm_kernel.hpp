@@ -1806,7 +1806,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   // adding, so the result does not depend on timing.  One block row of 32 rows at a time: NB * 4
   // groups of 16 bytes per lane and piece.
   if (DEPTH_PIECES && fix_pending) {
-    __syncthreads();   // (the description was written by the first thread)
+    __syncthreads();   // (the description was written by the first threads of the workgroup)
     int32_t words[kTileInfoDwords];
 #pragma unroll
     for (int i = 0; i < kTileInfoDwords; ++i) words[i] = sched->fix_tile[i];
