@@ -99,13 +99,18 @@ bool use_short_shape(int64_t num_groups, int64_t tokens, int trans_a) {
 // 256 groups around 256 rows -3.2 / -2.3 %, 96 around 256 -4.8 / -3.6 %, 128 around 512 -1.8 /
 // -2.2 %, around 768 -3.3 / -3.4 %, 64 around 1024 -1.2 / -1.6 %; around 128, 200, 320, 384, 640,
 // 1536, 2048 rows within +-0.7 %; Zipf sizes with groups of up to 57 tile rows +0.8 / +1.7 %
-// (hence the kernel's guard).  Small calls skip the second ranking pass (1-2 us).
+// (hence the kernel's guard).  It pays with deep tiles only: the same 256 groups around 256 rows
+// with hidden_in 4096 -2.6 / -1.9 %, 2048 +0.6 / -1.4 %, 1024 +1.6 / +0.7 %, 512 +8.9 / +7.4 %
+// (the order itself, a counting sort and a second scan of the tile counts, is 5-8 us of a launch
+// of 200 us there).
 constexpr int kByTileRowsGroups = 32;         // at least this many groups
 constexpr int kByTileRowsRowsBelow = 2048;    // ... of fewer rows than this on average
-constexpr int kByTileRowsRounds = 4;          // ... and at least this many rounds of tiles
+constexpr int kByTileRowsRounds = 4;          // ... at least this many rounds of tiles
+constexpr int kByTileRowsDepth = 2048;        // ... and tiles at least this deep
 
-bool order_by_tile_rows(int64_t num_groups, int64_t tokens, int64_t tiles_n, int bm, int grid) {
+bool order_by_tile_rows(int64_t num_groups, int64_t tokens, int64_t tiles_n, int bm, int grid, int64_t hidden_in) {
   return num_groups >= kByTileRowsGroups && tokens < (int64_t)kByTileRowsRowsBelow * num_groups &&
+         hidden_in >= kByTileRowsDepth &&
          (tokens / bm + num_groups / 2) * tiles_n >= (int64_t)kByTileRowsRounds * grid;
 }
 
@@ -421,7 +426,7 @@ int gmm_impl(const gg_gmm_args& g, bool static_scratch = false) {
     if (tiles == 0) continue;
     p.flags &= ~gg::kFlagByTileRows;
     if (!generic && !trans_a && !(p.flags & gg::kFlagGroupOrder) && count >= kByTileRowsGroups &&
-        order_by_tile_rows(num_groups, tokens, tiles_n, bm, info.cus))
+        order_by_tile_rows(num_groups, tokens, tiles_n, bm, info.cus, hidden_in))
       p.flags |= gg::kFlagByTileRows;
     // the full grid also for few tiles: the last round's tiles may be cut into pieces for
     // the workgroups that would otherwise idle
@@ -558,7 +563,7 @@ int gg_debug_schedule(const int64_t* batch_sizes, int batch_sizes_on_device, int
   {
     const int bm = short_shape ? Short::BM : Wide::BM, bn = short_shape ? Short::BN : Wide::BN;
     if (!trans_a && num_groups >= kByTileRowsGroups &&
-        order_by_tile_rows(num_groups, tokens, (hidden_out + bn - 1) / bn, bm, info.cus))
+        order_by_tile_rows(num_groups, tokens, (hidden_out + bn - 1) / bn, bm, info.cus, hidden_in))
       p.flags |= gg::kFlagByTileRows;
   }
   gg::HostSizes hs;

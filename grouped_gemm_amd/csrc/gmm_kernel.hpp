@@ -441,39 +441,33 @@ __device__ __forceinline__ void build_schedule(Sched* s, const GmmParams& p, con
   }
 }
 
-// Run by every thread of the workgroup after build_schedule and a barrier; ends with a barrier.
-// Fills Sched::order with the groups by descending key_of(group), groups of equal key in their
-// own order (what the reference's stable sort gives); `keys` is scratch for kMaxGroups 64-bit
+// Weight-gradient layout: the groups by descending depth, groups of equal depth in their own order
+// (what the reference's stable sort gives).  Run by every thread of the workgroup after
+// build_schedule and a barrier; ends with a barrier.  `keys` is scratch for kMaxGroups 64-bit
 // words (the tile buffers are not in use yet).
-template <typename KeyFn>
-__device__ __forceinline__ void order_groups(Sched* s, int num_groups, uint64_t* keys, KeyFn key_of) {
+__device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, uint64_t* keys) {
   // Up to a few hundred groups it is quicker to count, per group, the groups that go before it
-  // (measured equal at 256 groups, 12 us slower than the sort at 512).
+  // (measured equal at 256 groups, 12 us slower than the sort at 512): straight from
+  // Sched::rows, nothing written to `keys` (with the row counts copied there first the compiler
+  // built a different and 4-6 % slower depth loop for this layout).
   if (num_groups <= 256) {
-    // keys + 1, four to a 16-byte read (the same address in every lane: a broadcast), padded
-    // with zeros, which go before nothing
-    uint32_t* key32 = reinterpret_cast<uint32_t*>(keys);
-    const int padded = (num_groups + 3) & ~3;
-    for (int e = threadIdx.x; e < padded; e += blockDim.x) key32[e] = e < num_groups ? (uint32_t)key_of(e) + 1u : 0u;
-    __syncthreads();
     for (int e = threadIdx.x; e < num_groups; e += blockDim.x) {
-      const uint32_t mine = key32[e];
+      const int mine = s->rows[e];
       int before = 0;
-      for (int j = 0; j < padded; j += 4) {
-        const u32x4 other = *reinterpret_cast<const u32x4*>(key32 + j);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) before += (other[i] > mine || (other[i] == mine && j + i < e)) ? 1 : 0;
+      for (int j = 0; j < num_groups; ++j) {
+        const int other = s->rows[j];   // (the same address in every lane: a broadcast read)
+        before += (other > mine || (other == mine && j < e)) ? 1 : 0;
       }
       s->order[before] = (int16_t)e;
     }
     __syncthreads();
     return;
   }
-  // A bitonic sort in LDS of one 64-bit word per group, key above and 0xffff - index below.
+  // A bitonic sort in LDS of one 64-bit word per group, depth above and 0xffff - index below.
   int n = 2;
   while (n < num_groups) n <<= 1;
   for (int i = threadIdx.x; i < n; i += blockDim.x)
-    keys[i] = i < num_groups ? ((uint64_t)(uint32_t)key_of(i) << 16) | (uint64_t)(0xffff - i) : 0;   // padding sorts last
+    keys[i] = i < num_groups ? ((uint64_t)(uint32_t)s->rows[i] << 16) | (uint64_t)(0xffff - i) : 0;   // padding sorts last
   __syncthreads();
   for (int k = 2; k <= n; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
@@ -493,27 +487,6 @@ __device__ __forceinline__ void order_groups(Sched* s, int num_groups, uint64_t*
   }
   for (int i = threadIdx.x; i < num_groups; i += blockDim.x) s->order[i] = (int16_t)(0xffff - (int)(keys[i] & 0xffff));
   __syncthreads();
-}
-
-// Weight-gradient layout: the groups by descending depth.
-__device__ __forceinline__ void order_groups_by_depth(Sched* s, int num_groups, uint64_t* keys) {
-  // (the key is there already: counted straight from Sched::rows, nothing written to `keys`.  With
-  // the keys copied there first, as order_groups does, the compiler built a different and 4-6 %
-  // slower depth loop for this layout)
-  if (num_groups <= 256) {
-    for (int e = threadIdx.x; e < num_groups; e += blockDim.x) {
-      const int mine = s->rows[e];
-      int before = 0;
-      for (int j = 0; j < num_groups; ++j) {
-        const int other = s->rows[j];   // (the same address in every lane: a broadcast read)
-        before += (other > mine || (other == mine && j < e)) ? 1 : 0;
-      }
-      s->order[before] = (int16_t)e;
-    }
-    __syncthreads();
-    return;
-  }
-  order_groups(s, num_groups, keys, [&](int e) { return s->rows[e]; });
 }
 
 // Weight-gradient layout with a workspace, after order_groups_by_depth: tiles go out by descending
@@ -563,14 +536,57 @@ __device__ __forceinline__ void plan_deep_tiles(Sched* s, const GmmParams& p, in
 constexpr int kMaxTileRowsForOrder = 8;
 
 template <int LAYOUT, int BM, int BN>
-__device__ __forceinline__ void order_groups_by_tile_rows(Sched* s, const GmmParams& p, uint64_t* keys) {
+__device__ __forceinline__ void order_groups_by_tile_rows(Sched* s, const GmmParams& p) {
   const int E = p.num_groups;
-  if (s->most_rows > kMaxTileRowsForOrder * BM) {
-    for (int e = threadIdx.x; e < E; e += blockDim.x) s->order[e] = (int16_t)e;
-    __syncthreads();
-    return;
+  // A counting sort with one bucket per number of tile rows, by the first wave: each lane owns up
+  // to 8 consecutive groups, counts them by bucket, and one wave-wide scan per bucket gives every
+  // group its place (about a microsecond, where ranking the groups one against the other took 12).
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    const int per = (E + 63) >> 6;
+    const int e0 = lane * per;
+    if (s->most_rows > kMaxTileRowsForOrder * BM) {
+      for (int i = 0; i < per; ++i)
+        if (e0 + i < E) s->order[e0 + i] = (int16_t)(e0 + i);
+    } else {
+      constexpr int BUCKETS = kMaxTileRowsForOrder + 1;
+      int key[8], count[BUCKETS];
+#pragma unroll
+      for (int b = 0; b < BUCKETS; ++b) count[b] = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        key[i] = (i < per && e0 + i < E) ? (s->rows[e0 + i] + BM - 1) / BM : -1;
+#pragma unroll
+        for (int b = 0; b < BUCKETS; ++b) count[b] += key[i] == b ? 1 : 0;
+      }
+      int next[BUCKETS];   // where this lane's next group of a bucket goes
+      int base = 0;
+#pragma unroll
+      for (int b = 0; b < BUCKETS; ++b) {
+        int incl = count[b];
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int o = __shfl_up(incl, d);
+          if (lane >= d) incl += o;
+        }
+        next[b] = base + incl - count[b];
+        base += __shfl(incl, 63);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int at = -1;
+#pragma unroll
+        for (int b = 0; b < BUCKETS; ++b) {
+          if (key[i] == b) {
+            at = next[b];
+            next[b] += 1;
+          }
+        }
+        if (at >= 0) s->order[at] = (int16_t)(e0 + i);
+      }
+    }
   }
-  order_groups(s, E, keys, [&](int e) { return kMaxTileRowsForOrder - (s->rows[e] + BM - 1) / BM; });
+  __syncthreads();
   const int lane = threadIdx.x;
   if (lane < 64) {
     const int per = (E + 63) >> 6;
@@ -668,7 +684,7 @@ __global__ __launch_bounds__(64) void schedule_dump_kernel(GmmParams p, HostSize
   if (LAYOUT == kTN) {
     order_groups_by_depth(&s, p.num_groups, sort_keys);
   } else if (ordered) {
-    order_groups_by_tile_rows<LAYOUT, BM, BN>(&s, p, sort_keys);
+    order_groups_by_tile_rows<LAYOUT, BM, BN>(&s, p);
   }
   for (int e = threadIdx.x; e < p.num_groups; e += 64) {
     const GroupGeom g = group_geometry<LAYOUT>(p, p.first_group + e, s.row_start[e], s.rows[e]);
@@ -1276,7 +1292,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gmm_kernel(GmmParams p,
   if constexpr (LAYOUT == kTN) {
     order_groups_by_depth(sched, p.num_groups, reinterpret_cast<uint64_t*>(smem));
   } else {
-    if (p.flags & kFlagByTileRows) order_groups_by_tile_rows<LAYOUT, BM, BNS>(sched, p, reinterpret_cast<uint64_t*>(smem));
+    if (p.flags & kFlagByTileRows) order_groups_by_tile_rows<LAYOUT, BM, BNS>(sched, p);
   }
 
   const int lane = threadIdx.x & 63;

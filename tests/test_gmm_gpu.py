@@ -535,30 +535,36 @@ def test_c_abi_without_workspace_cuts_rows_bit_exactly(oracle):
 
 @pytest.mark.parametrize("trans_b", [False, True])
 def test_tiles_by_tile_rows_against_group_order(ops, oracle, trans_b):
-    # Many short groups of one, two and three tile rows: their tiles are handed out by ascending
-    # number of tile rows (see test_schedule_bit_exact for the order itself).  Every tile is computed as it
-    # would be in group order (shallow products: no depth pieces), so the outputs are equal bit for
-    # bit to those of GG_FLAG_GROUP_ORDER, and right against the oracle.  256 groups take the
-    # counting path of the ranking, 300 with empty ones the sorting path; device- and host-resident sizes.
-    cases = [([200 + (37 * i) % 180 for i in range(256)], 256, 1024),
-             ([0 if i % 7 == 0 else 100 + (53 * i) % 600 for i in range(300)], 192, 1032)]
+    # Many short groups of one, two and three tile rows, deep tiles: their tiles are handed out by
+    # ascending number of tile rows (see test_schedule_bit_exact for the order itself).  Every
+    # tile is computed as it would be in group order (no workspace: no depth pieces), so the
+    # outputs are equal bit for bit to those of GG_FLAG_GROUP_ORDER, and right against the oracle
+    # (on the first 40 groups: the whole product would keep the CPU busy for a quarter of a minute).
+    # With empty groups in the second case; device- and host-resident sizes.
+    lib = _c_abi()
+    cases = [([200 + (37 * i) % 180 for i in range(256)], 2048, 1024),
+             ([0 if i % 7 == 0 else 100 + (53 * i) % 600 for i in range(300)], 2056, 1032)]
     for idx, (sizes, hin, hout) in enumerate(cases):
         _announce("tiles by tile rows", trans_b, len(sizes), hin, hout)
         bs = torch.tensor(sizes, dtype=torch.int64)
         t = int(bs.sum())
-        assert _handed_out_by_tile_rows(sizes, -(-hout // 256), 256)
-        g = torch.Generator().manual_seed(40 + idx)
-        a = torch.randn(t, hin, generator=g).to(torch.bfloat16)
-        b = (torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g) * hin ** -0.5).to(torch.bfloat16)
-        da, db = a.cuda(), b.cuda()
+        assert _handed_out_by_tile_rows(sizes, hin, -(-hout // 256), 256)
+        g = torch.Generator(device="cuda").manual_seed(40 + idx)   # (operands of a gigabyte: made on the device)
+        da = torch.randn(t, hin, generator=g, device="cuda").to(torch.bfloat16)
+        db = (torch.randn(len(sizes), *((hout, hin) if trans_b else (hin, hout)), generator=g, device="cuda")
+              * hin ** -0.5).to(torch.bfloat16)
+        dbs = bs.cuda() if idx == 0 else bs
         by_tile_rows = torch.full((t + 1, hout), 7.0, dtype=torch.bfloat16, device="cuda")
-        ops.backend.backend.gmm(da, db, by_tile_rows[:t], bs.cuda() if idx == 0 else bs, False, trans_b)
+        args = _gmm_args(lib, da, db, by_tile_rows, dbs, idx == 0, t, hin, hout, False, trans_b)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
         in_order = torch.full((t + 1, hout), 7.0, dtype=torch.bfloat16, device="cuda")
-        ops.backend.backend.gmm_with_flags(da, db, in_order[:t], bs.cuda(), False, trans_b,
-                                           ops.backend.backend.flag_group_order)
+        args = _gmm_args(lib, da, db, in_order, dbs, idx == 0, t, hin, hout, False, trans_b, flags=8)
+        assert lib.gg_gmm(ctypes.byref(args)) == 0, lib.gg_last_error()
+        torch.cuda.synchronize()
         assert torch.equal(by_tile_rows, in_order)
         assert bool((by_tile_rows[t] == 7.0).all())
-        check(by_tile_rows[:t], oracle.gmm_loop(a, b, bs, trans_b=trans_b), f"case {idx}")
+        head = int(bs[:40].sum())
+        check(by_tile_rows[:head], oracle.gmm_loop(da[:head].cpu(), db[:40].cpu(), bs[:40], trans_b=trans_b), f"case {idx}")
 
 
 # ----------------------------------------------------------------- schedule, bit-exact
@@ -570,21 +576,22 @@ SCHED_CASES = [
     ([256] * 256, 7168, 2048),          # b offsets pass 2**31 elements
     ([1] * 512, 8, 8),
     ([70000, 0, 3, 70000], 2048, 1408),
-    # many short groups of one, two and three tile rows: handed out by their number of tile rows
-    # (NN and NT); 300 of them, with empty ones, take the sorting path of the ranking, 256 the
-    # counting one; the last case has one group of more than 8 tile rows and keeps the group order
+    # many short groups of one, two and three tile rows and deep tiles: handed out by their
+    # number of tile rows (NN and NT); with empty groups; with one group of more than 8 tile rows,
+    # which keeps the group order; with shallow tiles, which do too
     ([200 + (37 * i) % 180 for i in range(256)], 7168, 2048),
-    ([0 if i % 7 == 0 else 100 + (53 * i) % 600 for i in range(300)], 512, 1024),
-    ([2100 if i == 77 else 200 + (37 * i) % 180 for i in range(256)], 512, 2048),
+    ([0 if i % 7 == 0 else 100 + (53 * i) % 600 for i in range(300)], 2048, 1024),
+    ([2100 if i == 77 else 200 + (37 * i) % 180 for i in range(256)], 2048, 2048),
+    ([200 + (37 * i) % 180 for i in range(256)], 1024, 2048),
 ]
 
 
-def _handed_out_by_tile_rows(sizes, tiles_n, bm):
-    # the library's rule (gmm_api.hip, order_by_tile_rows): many groups, short on average, and enough
-    # tiles for several rounds; and the kernel's: no group of more than 8 tile rows
+def _handed_out_by_tile_rows(sizes, hin, tiles_n, bm):
+    # the library's rule (gmm_api.hip, order_by_tile_rows): many groups, short on average, deep
+    # tiles, and enough of them for several rounds; and the kernel's: no group of more than 8 tile rows
     grid = torch.cuda.get_device_properties(0).multi_processor_count
     num_groups, tokens = len(sizes), sum(sizes)
-    return (num_groups >= 32 and tokens < 2048 * num_groups and
+    return (num_groups >= 32 and tokens < 2048 * num_groups and hin >= 2048 and
             (tokens // bm + num_groups // 2) * tiles_n >= 4 * grid and max(sizes) <= 8 * bm)
 
 
@@ -622,7 +629,7 @@ def test_schedule_bit_exact(ops, oracle, sizes, hin, hout, layout, on_device):
         # NN and NT: in group order, or, for many short groups, by ascending number of tile rows,
         # groups of equal number in their own order; both prefix sums count in that order
         order = np.arange(len(sizes))
-        if _handed_out_by_tile_rows(sizes, -(-hout // bn.value), bm.value):
+        if _handed_out_by_tile_rows(sizes, hin, -(-hout // bn.value), bm.value):
             tile_rows = -(-np.array(sizes) // bm.value)
             order = np.argsort(tile_rows, kind="stable")
             if len(set(tile_rows.tolist())) > 2:
