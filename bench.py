@@ -34,10 +34,10 @@ PEAK_HBM_GBPS = 8000.0
 # the hash below (kernel_sources_sha16), and is reported only while the sources still have that
 # hash; the summary under profiles/ holds the figures, the commands and the commit.
 _TRAFFIC_KERNEL_SOURCES = ("gmm_kernel.hpp", "gmm_api.hip", "gmm_variants.hpp", "gmm_variants.def", "gmm_variant.hip")
-_TRAFFIC_KERNEL_SHA16 = "eaccfe62cdcea85f"
+_TRAFFIC_KERNEL_SHA16 = "7b530b46563c7867"
 _TRAFFIC_SOURCE = ("profiles/gmm_kernel_mixtral_w1_hbm_traffic.md and profiles/gmm_kernel_configs_3_4_5_stats_and_traffic.md "
                    "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources sha16 " + _TRAFFIC_KERNEL_SHA16 +
-                   ", commit b2b30cd; profiled once, not in this run)")
+                   ", commit 6d629b3; profiled once, not in this run)")
 
 
 def kernel_sources_sha16():
@@ -55,10 +55,10 @@ def _traffic(fetch_kib, write_kib):
 
 
 MEASURED_TRAFFIC = {
-    2: {"fwd": _traffic(4071720, 917560), "agrad": _traffic(3327540, 290023), "bgrad": _traffic(2752760, 917527)},
-    3: {"fwd": _traffic(423300, 135173)},
-    4: {"bgrad": _traffic(2756940, 917522)},
-    5: {"fwd": _traffic(4223150, 262209), "agrad": _traffic(4891020, 917545), "bgrad": _traffic(1851800, 7344580)},
+    2: {"fwd": _traffic(3987640, 917582), "agrad": _traffic(3327810, 289978), "bgrad": _traffic(2753890, 917538)},
+    3: {"fwd": _traffic(414260, 135176)},
+    4: {"bgrad": _traffic(2753050, 917541)},
+    5: {"fwd": _traffic(4225870, 262249), "agrad": _traffic(4955900, 917720), "bgrad": _traffic(1851750, 7344000)},
 }
 
 
